@@ -1,0 +1,170 @@
+/*
+ * polar_hip.h -- the thin C ABI between the PolarAI/Athena HIP runtime plugin
+ * (C++ host library, libpolar_rt_hip.so) and the gfx950 device code
+ * (libpolar_hip.so).
+ *
+ * Everything here is plain C: opaque handles, raw device pointers, 64-bit
+ * element counts.  All tensors are dense, row-major fp32, exactly as the
+ * reference's runtimes see them (src/backend/generic/runtime/sycl/kernels/
+ * common.hpp:35-38).  Kernel entry points enqueue work on the device's stream
+ * and return without waiting; ordering is stream order.
+ *
+ * Return value of every function that returns int: 0 on success, otherwise a
+ * polar_hip_status.  A message for the calling thread's last failure is kept
+ * and can be read with polar_hip_last_error().  The reference's convention for
+ * runtime failures is "print and terminate" (src/backend/generic/runtime/
+ * cuda/utils.hpp:20-28, hip/HIPContext.cpp:23-33); the C++ plugin above this
+ * layer applies it, this layer only reports.
+ *
+ * Each entry point names the reference interface it stands in for (paths
+ * relative to the reference tree).
+ */
+#ifndef POLAR_HIP_H
+#define POLAR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum polar_hip_status {
+  POLAR_HIP_OK = 0,
+  POLAR_HIP_ERR_INVALID = 1,   /* null pointer, bad shape, bad handle         */
+  POLAR_HIP_ERR_NO_DEVICE = 2, /* no usable gfx950 device / ordinal too large */
+  POLAR_HIP_ERR_OOM = 3,       /* device memory exhausted                     */
+  POLAR_HIP_ERR_RUNTIME = 4    /* a HIP call failed; see polar_hip_last_error */
+} polar_hip_status;
+
+typedef struct polar_hip_device polar_hip_device; /* one GPU: stream + pool  */
+typedef struct polar_hip_event polar_hip_event;   /* a point in stream order */
+
+typedef struct polar_hip_device_info {
+  char name[256];          /* marketing name                                  */
+  char arch[64];           /* gcnArchName, e.g. "gfx950:sramecc+:xnack-"      */
+  int ordinal;             /* HIP device ordinal                              */
+  int compute_units;       /* multiProcessorCount                             */
+  int clock_khz;           /* max engine clock                                */
+  int memory_clock_khz;    /* max memory clock                                */
+  int memory_bus_bits;     /* memory bus width                                */
+  int lds_bytes_per_block; /* sharedMemPerBlock                               */
+  int l2_bytes;            /* l2CacheSize                                     */
+  int pci_bus_id;
+  uint64_t hbm_bytes;      /* totalGlobalMem                                  */
+} polar_hip_device_info;
+
+typedef struct polar_hip_pool_stats {
+  uint64_t bytes_in_use;   /* handed out and not yet freed                    */
+  uint64_t bytes_cached;   /* held by the pool for reuse                      */
+  uint64_t device_allocs;  /* number of hipMalloc calls made so far           */
+  uint64_t pool_hits;      /* allocations served from cached blocks           */
+} polar_hip_pool_stats;
+
+const char* polar_hip_last_error(void);
+const char* polar_hip_version(void);
+
+/* ---- devices ---------------------------------------------------------------
+ * Stand in for device enumeration in the reference's contexts
+ * (src/backend/generic/runtime/hip/HIPContext.cpp:21-37,
+ *  src/backend/generic/runtime/sycl/SYCLContext.cpp:22-39). */
+int polar_hip_device_count(int* count);
+int polar_hip_device_open(int ordinal, polar_hip_device** out);
+int polar_hip_device_close(polar_hip_device* dev);
+int polar_hip_device_get_info(polar_hip_device* dev, polar_hip_device_info* out);
+/* Block the calling thread until everything enqueued on the device is done. */
+int polar_hip_device_synchronize(polar_hip_device* dev);
+
+/* ---- device memory pool -----------------------------------------------------
+ * Stand in for the per-tensor raw device allocation of the reference's
+ * allocator layers (src/backend/generic/runtime/cuda/CudaAllocator.hpp:54-78,
+ * src/backend/generic/runtime/sycl/USMAllocator.h:65-91).  Blocks are at least
+ * 256-byte aligned.  Freed blocks are cached and handed out again in stream
+ * order: a freed block may be reused by work enqueued later on the same
+ * device, never by work already enqueued. */
+int polar_hip_alloc(polar_hip_device* dev, uint64_t bytes, void** ptr);
+int polar_hip_free(polar_hip_device* dev, void* ptr);
+/* Return all cached blocks to the driver (waits for the stream first). */
+int polar_hip_pool_trim(polar_hip_device* dev);
+int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out);
+
+/* ---- host <-> device copies -------------------------------------------------
+ * Stand in for Device::copyToDevice / copyToHost of the reference's runtimes
+ * (src/backend/generic/runtime/cuda/CudaDevice.hpp:52-61,
+ *  src/backend/generic/runtime/sycl/SYCLDevice.h:81-112): ordered after all
+ * work already enqueued on the device, complete when the call returns. */
+int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
+                             const void* src_host, uint64_t bytes);
+int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
+                           const void* src_device, uint64_t bytes);
+
+/* ---- events -------------------------------------------------------------------
+ * Stand in for the native event inside the reference's Event objects
+ * (src/backend/generic/runtime/cuda/CudaEvent.cpp:18-31,
+ *  src/backend/generic/runtime/cuda/CudaDevice.cpp:109-113).  Events come from
+ * a per-device pool; release returns one to it. */
+int polar_hip_event_record(polar_hip_device* dev, polar_hip_event** out);
+int polar_hip_event_synchronize(polar_hip_event* evt);     /* host waits      */
+int polar_hip_event_query(polar_hip_event* evt, int* done); /* non-blocking   */
+/* Make later work on `dev` wait for `evt` (which may belong to another device)
+ * without blocking the host. */
+int polar_hip_stream_wait_event(polar_hip_device* dev, polar_hip_event* evt);
+/* Milliseconds between two completed events recorded on the same device. */
+int polar_hip_event_elapsed_ms(polar_hip_event* start, polar_hip_event* stop,
+                               float* ms);
+int polar_hip_event_release(polar_hip_event* evt);
+
+/* ---- builtin-operation kernels ---------------------------------------------
+ * One entry point per nativeKernelName the launch lowering can emit
+ * (utils/dialects/include/PolarGraph/PolarGraphOps.td:237,275,296,317,
+ *  343-351,371,393,481,523,542).  n counts elements.  Pointers are device
+ * pointers and may have any 4-byte alignment; output may alias an input only
+ * where the two are the same pointer (in-place). */
+
+/* fadd: c[i] = scaleA*a[i] + scaleB*b[i]
+ * (src/backend/generic/runtime/sycl/kernels/AddNaive.hpp:33-35) */
+int polar_hip_fadd(polar_hip_device* dev, const float* a, float scaleA,
+                   const float* b, float scaleB, float* c, uint64_t n);
+/* fmul: c[i] = a[i]*b[i]  (sycl/kernels/Mul.hpp:32) */
+int polar_hip_fmul(polar_hip_device* dev, const float* a, const float* b,
+                   float* c, uint64_t n);
+/* fdivide: out[i] = numerator[i]/denominator[i], IEEE rounding
+ * (sycl/kernels/Divide.hpp:33-35) */
+int polar_hip_fdivide(polar_hip_device* dev, const float* numerator,
+                      const float* denominator, float* out, uint64_t n);
+/* fsigmoid: 1/(1+exp(-x)) clamped into [1e-5, 1-1e-5]
+ * (sycl/kernels/Sigmoid.hpp:32-41) */
+int polar_hip_fsigmoid(polar_hip_device* dev, const float* in, float* out,
+                       uint64_t n);
+/* flogloss: -g*log(p+1e-5) - (1-g)*log(1-p+1e-5), elementwise
+ * (sycl/kernels/LogLoss.hpp:33-37) */
+int polar_hip_flogloss(polar_hip_device* dev, const float* predicted,
+                       const float* groundTruth, float* out, uint64_t n);
+/* fmulconcat: out[i] = gradient[0]*localDerivative[i]
+ * (sycl/kernels/MulConcat.hpp:33-35) */
+int polar_hip_fmulconcat(polar_hip_device* dev, const float* gradient,
+                         const float* localDerivative, float* out, uint64_t n);
+/* fcopy: dst = src (sycl/kernels/Copy.hpp:27-57) */
+int polar_hip_fcopy(polar_hip_device* dev, const float* src, float* dst,
+                    uint64_t n);
+/* ffill: out[i] = pattern (sycl/kernels/Fill.hpp:54-81) */
+int polar_hip_ffill(polar_hip_device* dev, float pattern, float* out,
+                    uint64_t n);
+/* ftranspose: out[j*rows+i] = in[i*cols+j]; in is rows x cols
+ * (spec only: include/polarai/core/internal/GenBuiltins.hpp:50,
+ *  utils/dialects/include/PolarGraph/PolarGraphOps.td:507-527) */
+int polar_hip_ftranspose(polar_hip_device* dev, const float* in, float* out,
+                         uint64_t rows, uint64_t cols);
+/* fmatmul_{f,t}_{f,t}: C[M x N] = opA(A) * opB(B), C overwritten, fp32.
+ * A is stored [M x K] (transA = 0) or [K x M] (transA != 0); B is stored
+ * [K x N] (transB = 0) or [N x K] (transB != 0)
+ * (sycl/kernels/MatMul.hpp:33-64; shapes as in
+ *  tests/integration/operations/MatMulOperation.cpp:203-204,249-250). */
+int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
+                      const float* a, const float* b, float* c, uint64_t m,
+                      uint64_t n, uint64_t k);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* POLAR_HIP_H */

@@ -1,0 +1,268 @@
+// Memory-bound builtin operations for gfx950: fadd fmul fdivide fsigmoid
+// flogloss fmulconcat fcopy ffill.
+//
+// One kernel template serves all of them.  A work-group of 256 lanes owns a
+// tile of 256*UNROLL 16-byte vectors; every lane issues all of its dwordx4
+// loads before the first use so that UNROLL*NIN loads per lane are in flight,
+// then computes and stores.  Loads and stores are marked non-temporal: every
+// byte is touched once, so keeping it in L2 / Infinity Cache only evicts other
+// data.  Tiles are handed out grid-stride so any element count fits the grid.
+// The n % 4 trailing elements are done by the first lanes of block 0.  Buffers
+// that are not 16-byte aligned take a dword kernel instead.
+//
+// Arithmetic is written so that it rounds exactly like the host kernels it
+// replaces: this file is compiled with -ffp-contract=off (no fused
+// multiply-add in `sa*a + sb*b`), `/` is the correctly rounded IEEE division
+// and expf/logf are the full-precision library versions.
+#include "internal.h"
+
+using namespace polar_hip_detail;
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kBlock = 256;
+
+// ---- per-element operations ---------------------------------------------------
+// NIN = number of input streams.  apply(x, y) receives the i-th element of each.
+
+struct AddOp { // src/backend/generic/runtime/sycl/kernels/AddNaive.hpp:33-35
+  static constexpr int NIN = 2;
+  float sa, sb;
+  __device__ __forceinline__ float apply(float a, float b) const {
+    return sa * a + sb * b;
+  }
+};
+struct MulOp { // sycl/kernels/Mul.hpp:32
+  static constexpr int NIN = 2;
+  __device__ __forceinline__ float apply(float a, float b) const {
+    return a * b;
+  }
+};
+struct DivOp { // sycl/kernels/Divide.hpp:33-35
+  static constexpr int NIN = 2;
+  __device__ __forceinline__ float apply(float a, float b) const {
+    return a / b;
+  }
+};
+struct LogLossOp { // sycl/kernels/LogLoss.hpp:33-37
+  static constexpr int NIN = 2;
+  __device__ __forceinline__ float apply(float p, float g) const {
+    const float eps = 1e-5f;
+    return -g * logf(p + eps) - (1.0f - g) * logf(1.0f - p + eps);
+  }
+};
+struct SigmoidOp { // sycl/kernels/Sigmoid.hpp:32-41
+  static constexpr int NIN = 1;
+  __device__ __forceinline__ float apply(float x, float) const {
+    const float eps = 1e-5f;
+    float r = 1.0f / (1.0f + expf(-x));
+    if (fabsf(r - 1.0f) < eps) {
+      r = 1.0f - eps;
+    } else if (fabsf(r) < eps) {
+      r = eps;
+    }
+    return r;
+  }
+};
+struct ScaleOp { // sycl/kernels/MulConcat.hpp:33-35 (g = gradient[0])
+  static constexpr int NIN = 1;
+  float g;
+  __device__ __forceinline__ float apply(float d, float) const {
+    return g * d;
+  }
+};
+struct CopyOp { // sycl/kernels/Copy.hpp:49-53
+  static constexpr int NIN = 1;
+  __device__ __forceinline__ float apply(float s, float) const { return s; }
+};
+struct FillOp { // sycl/kernels/Fill.hpp:69-74
+  static constexpr int NIN = 0;
+  float pattern;
+  __device__ __forceinline__ float apply(float, float) const {
+    return pattern;
+  }
+};
+
+template <typename Op>
+__device__ __forceinline__ v4f apply4(const Op& op, v4f a, v4f b) {
+  v4f r;
+  r.x = op.apply(a.x, b.x);
+  r.y = op.apply(a.y, b.y);
+  r.z = op.apply(a.z, b.z);
+  r.w = op.apply(a.w, b.w);
+  return r;
+}
+
+// fmulconcat reads its scalar from device memory; every lane reads the same
+// address, which the compiler turns into one scalar load per wave.
+template <typename Op> struct OpLoader {
+  __device__ static Op load(const Op& op, const float*) { return op; }
+};
+template <> struct OpLoader<ScaleOp> {
+  __device__ static ScaleOp load(const ScaleOp&, const float* g) {
+    return ScaleOp{g[0]};
+  }
+};
+
+template <typename Op, int UNROLL>
+__global__ __launch_bounds__(kBlock) void ewVecKernel(
+    Op op0, const float* scalarSrc, const v4f* a, const v4f* b, v4f* c,
+    uint64_t n4, uint64_t n, uint64_t numTiles) {
+  const Op op = OpLoader<Op>::load(op0, scalarSrc);
+  constexpr uint64_t kTile = uint64_t(kBlock) * UNROLL;
+  for (uint64_t tile = blockIdx.x; tile < numTiles; tile += gridDim.x) {
+    const uint64_t base = tile * kTile + threadIdx.x;
+    v4f va[UNROLL], vb[UNROLL];
+    if (base - threadIdx.x + kTile <= n4) { // whole tile in range
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t i = base + uint64_t(u) * kBlock;
+        va[u] = Op::NIN >= 1 ? __builtin_nontemporal_load(&a[i]) : v4f{0, 0, 0, 0};
+        vb[u] = Op::NIN >= 2 ? __builtin_nontemporal_load(&b[i]) : v4f{0, 0, 0, 0};
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t i = base + uint64_t(u) * kBlock;
+        __builtin_nontemporal_store(apply4(op, va[u], vb[u]), &c[i]);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t i = base + uint64_t(u) * kBlock;
+        if (i < n4) {
+          va[u] = Op::NIN >= 1 ? __builtin_nontemporal_load(&a[i]) : v4f{0, 0, 0, 0};
+          vb[u] = Op::NIN >= 2 ? __builtin_nontemporal_load(&b[i]) : v4f{0, 0, 0, 0};
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint64_t i = base + uint64_t(u) * kBlock;
+        if (i < n4) __builtin_nontemporal_store(apply4(op, va[u], vb[u]), &c[i]);
+      }
+    }
+  }
+  // trailing n % 4 elements
+  if (blockIdx.x == 0) {
+    const uint64_t i = n4 * 4 + threadIdx.x;
+    if (i < n) {
+      const float* as = reinterpret_cast<const float*>(a);
+      const float* bs = reinterpret_cast<const float*>(b);
+      float x = Op::NIN >= 1 ? as[i] : 0.0f;
+      float y = Op::NIN >= 2 ? bs[i] : 0.0f;
+      reinterpret_cast<float*>(c)[i] = op.apply(x, y);
+    }
+  }
+}
+
+// Buffers with only 4-byte alignment: one dword per lane per step.
+template <typename Op>
+__global__ __launch_bounds__(kBlock) void ewScalarKernel(
+    Op op0, const float* scalarSrc, const float* a, const float* b, float* c,
+    uint64_t n) {
+  const Op op = OpLoader<Op>::load(op0, scalarSrc);
+  const uint64_t stride = uint64_t(gridDim.x) * kBlock;
+  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < n;
+       i += stride) {
+    float x = Op::NIN >= 1 ? a[i] : 0.0f;
+    float y = Op::NIN >= 2 ? b[i] : 0.0f;
+    c[i] = op.apply(x, y);
+  }
+}
+
+template <typename Op, int UNROLL>
+int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
+             const float* a, const float* b, float* c, uint64_t n) {
+  if (n == 0) return POLAR_HIP_OK;
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  const bool vec = aligned16(c) && (Op::NIN < 1 || aligned16(a)) &&
+                   (Op::NIN < 2 || aligned16(b));
+  if (vec) {
+    const uint64_t n4 = n / 4;
+    constexpr uint64_t kTile = uint64_t(kBlock) * UNROLL;
+    const uint64_t numTiles = (n4 + kTile - 1) / kTile;
+    uint64_t grid = numTiles < 1 ? 1 : numTiles;
+    if (grid > (1u << 22)) grid = 1u << 22;
+    ewVecKernel<Op, UNROLL><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
+                              dev->stream>>>(
+        op, scalarSrc, reinterpret_cast<const v4f*>(a),
+        reinterpret_cast<const v4f*>(b), reinterpret_cast<v4f*>(c), n4, n,
+        numTiles);
+  } else {
+    uint64_t grid = (n + kBlock - 1) / kBlock;
+    const uint64_t cap = uint64_t(dev->info.compute_units) * 32;
+    if (grid > cap) grid = cap;
+    ewScalarKernel<Op><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
+                         dev->stream>>>(op, scalarSrc, a, b, c, n);
+  }
+  POLAR_HIP_TRY(hipGetLastError());
+  return POLAR_HIP_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int polar_hip_fadd(polar_hip_device* dev, const float* a, float scaleA,
+                   const float* b, float scaleB, float* c, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (a && b && c), "null tensor");
+  return launchEw<AddOp, 4>(dev, AddOp{scaleA, scaleB}, nullptr, a, b, c, n);
+}
+
+int polar_hip_fmul(polar_hip_device* dev, const float* a, const float* b,
+                   float* c, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (a && b && c), "null tensor");
+  return launchEw<MulOp, 4>(dev, MulOp{}, nullptr, a, b, c, n);
+}
+
+int polar_hip_fdivide(polar_hip_device* dev, const float* numerator,
+                      const float* denominator, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (numerator && denominator && out), "null tensor");
+  return launchEw<DivOp, 4>(dev, DivOp{}, nullptr, numerator, denominator, out,
+                            n);
+}
+
+int polar_hip_fsigmoid(polar_hip_device* dev, const float* in, float* out,
+                       uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (in && out), "null tensor");
+  return launchEw<SigmoidOp, 4>(dev, SigmoidOp{}, nullptr, in, nullptr, out, n);
+}
+
+int polar_hip_flogloss(polar_hip_device* dev, const float* predicted,
+                       const float* groundTruth, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (predicted && groundTruth && out), "null tensor");
+  return launchEw<LogLossOp, 4>(dev, LogLossOp{}, nullptr, predicted,
+                                groundTruth, out, n);
+}
+
+int polar_hip_fmulconcat(polar_hip_device* dev, const float* gradient,
+                         const float* localDerivative, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (gradient && localDerivative && out),
+                    "null tensor");
+  return launchEw<ScaleOp, 4>(dev, ScaleOp{0.0f}, gradient, localDerivative,
+                              nullptr, out, n);
+}
+
+int polar_hip_fcopy(polar_hip_device* dev, const float* src, float* dst,
+                    uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (src && dst), "null tensor");
+  return launchEw<CopyOp, 4>(dev, CopyOp{}, nullptr, src, nullptr, dst, n);
+}
+
+int polar_hip_ffill(polar_hip_device* dev, float pattern, float* out,
+                    uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || out, "null tensor");
+  return launchEw<FillOp, 4>(dev, FillOp{pattern}, nullptr, nullptr, nullptr,
+                             out, n);
+}
+
+} // extern "C"

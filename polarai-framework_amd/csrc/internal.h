@@ -1,0 +1,60 @@
+// Shared definitions of the device library: the device handle (stream, memory
+// pool, event pool), error reporting and launch helpers.  Not installed; the
+// public surface is include/polar_hip.h.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "polar_hip.h"
+
+struct polar_hip_event {
+  polar_hip_device* dev;
+  hipEvent_t ev;
+};
+
+struct polar_hip_device {
+  int ordinal = 0;
+  hipStream_t stream = nullptr;
+  polar_hip_device_info info{};
+
+  std::mutex mu;
+  // pool: rounded block size -> cached blocks; live block -> rounded size
+  std::map<uint64_t, std::vector<void*>> cached;
+  std::unordered_map<void*, uint64_t> live;
+  polar_hip_pool_stats stats{};
+  std::vector<polar_hip_event*> idleEvents;
+  std::vector<polar_hip_event*> allEvents;
+
+};
+
+namespace polar_hip_detail {
+
+int fail(polar_hip_status st, const char* fmt, ...)
+    __attribute__((format(printf, 2, 3)));
+int failHip(hipError_t e, const char* what);
+
+inline bool aligned16(const void* p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+} // namespace polar_hip_detail
+
+#define POLAR_HIP_TRY(expr)                                                    \
+  do {                                                                         \
+    hipError_t e_ = (expr);                                                    \
+    if (e_ != hipSuccess) return polar_hip_detail::failHip(e_, #expr);        \
+  } while (0)
+
+#define POLAR_HIP_REQUIRE(cond, msg)                                           \
+  do {                                                                         \
+    if (!(cond))                                                               \
+      return polar_hip_detail::fail(POLAR_HIP_ERR_INVALID, "%s: %s", __func__, \
+                                    msg);                                      \
+  } while (0)

@@ -1,0 +1,309 @@
+// fmatmul_{f,t}_{f,t} for gfx950: C[M x N] = opA(A) * opB(B), fp32 in, fp32
+// accumulate, C overwritten.
+//
+// The contraction runs on the matrix cores with v_mfma_f32_32x32x2_f32 (true
+// fp32; gfx950 has no reduced-precision fp32 matrix path).  A work-group owns a
+// BM x BN tile of C and walks K in steps of BK.  Both operand tiles are staged
+// in LDS k-major (S[k][x], x = row of C for A, column of C for B) whatever the
+// storage order in HBM, so the four transpose variants differ only in how a
+// tile is fetched:
+//   * operand contiguous along k (A not transposed, B transposed): a lane
+//     loads 4 consecutive k of one row and scatters them to 4 LDS rows;
+//   * operand contiguous along x (A transposed, B not transposed): a lane
+//     loads 4 consecutive x of one k and stores them as one 16-byte LDS write.
+// The next tile is fetched into registers while the current one is multiplied
+// (two LDS stages, one barrier per step).  Each wave owns a (BM/WM) x (BN/WN)
+// sub-tile as TM x TN accumulator blocks of 32x32; per k-pair it reads TM + TN
+// LDS words per lane and issues TM*TN MFMAs.  LDS row pitch is BX + 4 words so
+// the scattered stores of the k-contiguous case spread over the banks.
+//
+// Work-groups are numbered so that the groups resident on one XCD (which share
+// an L2) cover a compact block of C tiles and therefore re-use the same rows
+// of A and columns of B.
+//
+// Shapes that are not multiples of the tile, leading dimensions that are not
+// multiples of 4 and unaligned base pointers are handled by predicated /
+// scalar fetch variants chosen on the host.
+#include "internal.h"
+
+using namespace polar_hip_detail;
+
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kLdsPad = 4;
+constexpr int kXcds = 8;
+
+struct MatmulArgs {
+  const float* A;
+  const float* B;
+  float* C;
+  uint32_t M, N, K;
+  uint32_t tilesM, tilesN;
+};
+
+// Fetch of one operand tile (BX x BK) from HBM into registers, and its store
+// into the k-major LDS stage.  KCONTIG: element (x, k) lives at
+// X[(x0+x)*ld + k0+k]; otherwise at X[(k0+k)*ld + x0+x].
+template <int BX, int BK, int NT, bool KCONTIG, bool VEC, bool EDGE>
+struct TileFetch {
+  static constexpr int kVecs = BX * BK / 4 / NT;  // 16-byte loads per lane
+  static constexpr int kScalars = BX * BK / NT;   // dword loads per lane
+  static_assert(BX * BK % (4 * NT) == 0, "tile must divide over the lanes");
+  float r[kScalars];
+
+  __device__ __forceinline__ void load(const float* X, size_t ld, uint32_t x0,
+                                       uint32_t k0, uint32_t xdim,
+                                       uint32_t kdim, int t) {
+    if constexpr (VEC) {
+#pragma unroll
+      for (int v = 0; v < kVecs; ++v) {
+        const int vid = t + v * NT;
+        uint32_t x, k;
+        if constexpr (KCONTIG) {
+          x = vid / (BK / 4);
+          k = (vid % (BK / 4)) * 4;
+        } else {
+          k = vid / (BX / 4);
+          x = (vid % (BX / 4)) * 4;
+        }
+        const size_t off = KCONTIG ? size_t(x0 + x) * ld + (k0 + k)
+                                   : size_t(k0 + k) * ld + (x0 + x);
+        v4f g;
+        if (!EDGE || (x0 + x < xdim && k0 + k < kdim)) {
+          g = *reinterpret_cast<const v4f*>(X + off);
+        } else {
+          g = v4f{0.f, 0.f, 0.f, 0.f};
+        }
+        r[4 * v + 0] = g.x;
+        r[4 * v + 1] = g.y;
+        r[4 * v + 2] = g.z;
+        r[4 * v + 3] = g.w;
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < kScalars; ++s) {
+        const int sid = t + s * NT;
+        uint32_t x, k;
+        if constexpr (KCONTIG) {
+          x = sid / BK;
+          k = sid % BK;
+        } else {
+          k = sid / BX;
+          x = sid % BX;
+        }
+        const size_t off = KCONTIG ? size_t(x0 + x) * ld + (k0 + k)
+                                   : size_t(k0 + k) * ld + (x0 + x);
+        r[s] = (!EDGE || (x0 + x < xdim && k0 + k < kdim)) ? X[off] : 0.f;
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(float* S, int t) const {
+    constexpr int LD = BX + kLdsPad;
+    if constexpr (VEC) {
+#pragma unroll
+      for (int v = 0; v < kVecs; ++v) {
+        const int vid = t + v * NT;
+        if constexpr (KCONTIG) {
+          const int x = vid / (BK / 4);
+          const int k = (vid % (BK / 4)) * 4;
+#pragma unroll
+          for (int c = 0; c < 4; ++c) S[(k + c) * LD + x] = r[4 * v + c];
+        } else {
+          const int k = vid / (BX / 4);
+          const int x = (vid % (BX / 4)) * 4;
+          *reinterpret_cast<v4f*>(&S[k * LD + x]) =
+              v4f{r[4 * v], r[4 * v + 1], r[4 * v + 2], r[4 * v + 3]};
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < kScalars; ++s) {
+        const int sid = t + s * NT;
+        const int x = KCONTIG ? sid / BK : sid % BX;
+        const int k = KCONTIG ? sid % BK : sid / BX;
+        S[k * LD + x] = r[s];
+      }
+    }
+  }
+};
+
+// Linear work-group id -> C tile, such that the groups an XCD receives
+// (ids congruent modulo 8) are consecutive in a panel-major walk over C.
+__device__ __forceinline__ void tileOfGroup(uint32_t bid, uint32_t nGroups,
+                                            uint32_t tilesM, uint32_t tilesN,
+                                            uint32_t& tm, uint32_t& tn) {
+  uint32_t lin = bid;
+  if (nGroups % kXcds == 0) lin = (bid % kXcds) * (nGroups / kXcds) + bid / kXcds;
+  constexpr uint32_t kPanel = 8; // tile rows walked together
+  const uint32_t perPanel = kPanel * tilesN;
+  const uint32_t panel = lin / perPanel;
+  const uint32_t first = panel * kPanel;
+  const uint32_t rows = tilesM - first < kPanel ? tilesM - first : kPanel;
+  const uint32_t in = lin % perPanel;
+  tm = first + in % rows;
+  tn = in / rows;
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB, bool VEC,
+          bool EDGE>
+__global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN;
+  constexpr int TM = WTM / 32, TN = WTN / 32;
+  constexpr int LDA = BM + kLdsPad, LDB = BN + kLdsPad;
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32");
+  static_assert(BK % 4 == 0, "BK multiple of 4");
+
+  __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
+  __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
+
+  const int t = threadIdx.x;
+  const int lane = t % 64;
+  const int wave = t / 64;
+  const int wm = wave / WN, wn = wave % WN;
+
+  uint32_t tm, tn;
+  tileOfGroup(blockIdx.x, gridDim.x, p.tilesM, p.tilesN, tm, tn);
+  const uint32_t m0 = tm * BM, n0 = tn * BN;
+
+  // A: k-contiguous when not transposed ([M x K]); B: k-contiguous when
+  // transposed ([N x K]).
+  TileFetch<BM, BK, NT, !TA, VEC, EDGE> fa;
+  TileFetch<BN, BK, NT, TB, VEC, EDGE> fb;
+  const size_t lda = TA ? p.M : p.K;
+  const size_t ldb = TB ? p.K : p.N;
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const uint32_t nk = (p.K + BK - 1) / BK;
+  fa.load(p.A, lda, m0, 0, p.M, p.K, t);
+  fb.load(p.B, ldb, n0, 0, p.N, p.K, t);
+  fa.store(As[0], t);
+  fb.store(Bs[0], t);
+  __syncthreads();
+
+  const int aBase = wm * WTM + (lane % 32);
+  const int bBase = wn * WTN + (lane % 32);
+  const int kLane = lane / 32;
+
+  for (uint32_t kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    const bool more = kt + 1 < nk;
+    if (more) {
+      fa.load(p.A, lda, m0, (kt + 1) * BK, p.M, p.K, t);
+      fb.load(p.B, ldb, n0, (kt + 1) * BK, p.N, p.K, t);
+    }
+    const float* as = As[cur];
+    const float* bs = Bs[cur];
+#pragma unroll
+    for (int kk = 0; kk < BK; kk += 2) {
+      float a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = as[(kk + kLane) * LDA + aBase + i * 32];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) b[j] = bs[(kk + kLane) * LDB + bBase + j * 32];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j],
+                                                          0, 0, 0);
+    }
+    if (more) {
+      fa.store(As[cur ^ 1], t);
+      fb.store(Bs[cur ^ 1], t);
+    }
+    __syncthreads();
+  }
+
+  // Accumulator block layout of the 32x32 MFMA: register r of lane l holds
+  // row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const uint32_t col = n0 + wn * WTN + j * 32 + (lane % 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t row =
+            m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
+        if (!EDGE || (row < p.M && col < p.N))
+          p.C[size_t(row) * p.N + col] = acc[i][j][r];
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
+int launchLayout(polar_hip_device* dev, const MatmulArgs& p0, bool vec,
+                 bool edge) {
+  MatmulArgs p = p0;
+  p.tilesM = (p.M + BM - 1) / BM;
+  p.tilesN = (p.N + BN - 1) / BN;
+  const uint64_t groups = uint64_t(p.tilesM) * p.tilesN;
+  if (groups >= (1ull << 31))
+    return fail(POLAR_HIP_ERR_INVALID, "fmatmul: too many tiles");
+  const dim3 grid(static_cast<unsigned>(groups)), block(WM * WN * 64);
+  if (vec && !edge)
+    matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, false>
+        <<<grid, block, 0, dev->stream>>>(p);
+  else if (vec && edge)
+    matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, true>
+        <<<grid, block, 0, dev->stream>>>(p);
+  else
+    matmulKernel<BM, BN, BK, WM, WN, TA, TB, false, true>
+        <<<grid, block, 0, dev->stream>>>(p);
+  POLAR_HIP_TRY(hipGetLastError());
+  return POLAR_HIP_OK;
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p) {
+  // 16-byte fetches need aligned bases and a contiguous dimension that is a
+  // multiple of 4 for both operands.
+  const uint32_t contigA = ta ? p.M : p.K;
+  const uint32_t contigB = tb ? p.K : p.N;
+  const bool vec = aligned16(p.A) && aligned16(p.B) && contigA % 4 == 0 &&
+                   contigB % 4 == 0;
+  const bool edge = p.M % BM != 0 || p.N % BN != 0 || p.K % BK != 0;
+  if (!ta && !tb) return launchLayout<BM, BN, BK, WM, WN, false, false>(dev, p, vec, edge);
+  if (!ta && tb) return launchLayout<BM, BN, BK, WM, WN, false, true>(dev, p, vec, edge);
+  if (ta && !tb) return launchLayout<BM, BN, BK, WM, WN, true, false>(dev, p, vec, edge);
+  return launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
+}
+
+} // namespace
+
+extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
+                                 const float* a, const float* b, float* c,
+                                 uint64_t m, uint64_t n, uint64_t k) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  if (m == 0 || n == 0) return POLAR_HIP_OK;
+  POLAR_HIP_REQUIRE(c != nullptr, "null output");
+  POLAR_HIP_REQUIRE(k == 0 || (a != nullptr && b != nullptr), "null operand");
+  POLAR_HIP_REQUIRE(m < (1ull << 31) && n < (1ull << 31) && k < (1ull << 31),
+                    "dimension does not fit 31 bits");
+  POLAR_HIP_REQUIRE(c != a && c != b, "output aliases an operand");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  if (k == 0) {
+    // Empty contraction: the reference's loop leaves acc = 0 and stores it.
+    return polar_hip_ffill(dev, 0.0f, c, m * n);
+  }
+  MatmulArgs p{a, b, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+               static_cast<uint32_t>(k), 0, 0};
+  const bool ta = transA != 0, tb = transB != 0;
+  if (n <= 32) return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p);
+  if (m <= 32) return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p);
+  if (m <= 64 || n <= 64) return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p);
+  return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p);
+}

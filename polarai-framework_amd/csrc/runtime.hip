@@ -1,0 +1,308 @@
+// Device handle, memory pool, host<->device copies and events of the device
+// library (the non-kernel half of include/polar_hip.h).
+#include "internal.h"
+
+#include <cstdio>
+#include <cstring>
+
+namespace {
+thread_local char g_lastError[512] = "";
+
+uint64_t roundBlock(uint64_t bytes) {
+  // Small blocks: powers of two from 256 B.  Large blocks: multiples of 2 MiB,
+  // so that tensors of nearly equal size share cached blocks.
+  if (bytes <= 256) return 256;
+  if (bytes <= (1ull << 20)) {
+    uint64_t r = 256;
+    while (r < bytes) r <<= 1;
+    return r;
+  }
+  const uint64_t g = 2ull << 20;
+  return (bytes + g - 1) / g * g;
+}
+} // namespace
+
+namespace polar_hip_detail {
+int fail(polar_hip_status st, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_lastError, sizeof(g_lastError), fmt, ap);
+  va_end(ap);
+  return static_cast<int>(st);
+}
+int failHip(hipError_t e, const char* what) {
+  polar_hip_status st = e == hipErrorOutOfMemory ? POLAR_HIP_ERR_OOM
+                        : e == hipErrorNoDevice  ? POLAR_HIP_ERR_NO_DEVICE
+                                                 : POLAR_HIP_ERR_RUNTIME;
+  return fail(st, "%s failed: %s (%d)", what, hipGetErrorString(e),
+              static_cast<int>(e));
+}
+} // namespace polar_hip_detail
+
+using namespace polar_hip_detail;
+
+extern "C" {
+
+const char* polar_hip_last_error(void) { return g_lastError; }
+const char* polar_hip_version(void) { return "polar_hip 0.1 (gfx950)"; }
+
+int polar_hip_device_count(int* count) {
+  POLAR_HIP_REQUIRE(count != nullptr, "count is null");
+  *count = 0;
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e == hipErrorNoDevice) {
+    (void)hipGetLastError();
+    return POLAR_HIP_OK;
+  }
+  if (e != hipSuccess) return failHip(e, "hipGetDeviceCount");
+  *count = n;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_device_open(int ordinal, polar_hip_device** out) {
+  POLAR_HIP_REQUIRE(out != nullptr, "out is null");
+  *out = nullptr;
+  int n = 0;
+  int st = polar_hip_device_count(&n);
+  if (st) return st;
+  if (ordinal < 0 || ordinal >= n)
+    return fail(POLAR_HIP_ERR_NO_DEVICE, "device ordinal %d of %d", ordinal, n);
+  POLAR_HIP_TRY(hipSetDevice(ordinal));
+  hipDeviceProp_t p;
+  POLAR_HIP_TRY(hipGetDeviceProperties(&p, ordinal));
+  if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+    return fail(POLAR_HIP_ERR_NO_DEVICE,
+                "device %d is %s; this library holds gfx950 code only", ordinal,
+                p.gcnArchName);
+  auto* d = new polar_hip_device();
+  d->ordinal = ordinal;
+  hipError_t e = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    delete d;
+    return failHip(e, "hipStreamCreateWithFlags");
+  }
+  snprintf(d->info.name, sizeof(d->info.name), "%s", p.name);
+  snprintf(d->info.arch, sizeof(d->info.arch), "%s", p.gcnArchName);
+  d->info.ordinal = ordinal;
+  d->info.compute_units = p.multiProcessorCount;
+  d->info.clock_khz = p.clockRate;
+  d->info.memory_clock_khz = p.memoryClockRate;
+  d->info.memory_bus_bits = p.memoryBusWidth;
+  d->info.lds_bytes_per_block = static_cast<int>(p.sharedMemPerBlock);
+  d->info.l2_bytes = p.l2CacheSize;
+  d->info.pci_bus_id = p.pciBusID;
+  d->info.hbm_bytes = p.totalGlobalMem;
+  *out = d;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_device_close(polar_hip_device* dev) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  for (auto& kv : dev->cached)
+    for (void* p : kv.second) (void)hipFree(p);
+  for (auto& kv : dev->live) (void)hipFree(kv.first);
+  for (auto* e : dev->allEvents) {
+    (void)hipEventDestroy(e->ev);
+    delete e;
+  }
+  (void)hipStreamDestroy(dev->stream);
+  delete dev;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_device_get_info(polar_hip_device* dev,
+                              polar_hip_device_info* out) {
+  POLAR_HIP_REQUIRE(dev != nullptr && out != nullptr, "null argument");
+  *out = dev->info;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_device_synchronize(polar_hip_device* dev) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return POLAR_HIP_OK;
+}
+
+// ---- pool -------------------------------------------------------------------
+
+static void dropCachedLocked(polar_hip_device* dev) {
+  for (auto& kv : dev->cached)
+    for (void* p : kv.second) (void)hipFree(p);
+  dev->cached.clear();
+  dev->stats.bytes_cached = 0;
+}
+
+int polar_hip_alloc(polar_hip_device* dev, uint64_t bytes, void** ptr) {
+  POLAR_HIP_REQUIRE(dev != nullptr && ptr != nullptr, "null argument");
+  *ptr = nullptr;
+  const uint64_t sz = roundBlock(bytes);
+  std::lock_guard<std::mutex> g(dev->mu);
+  auto it = dev->cached.find(sz);
+  if (it != dev->cached.end() && !it->second.empty()) {
+    void* p = it->second.back();
+    it->second.pop_back();
+    dev->stats.bytes_cached -= sz;
+    dev->stats.bytes_in_use += sz;
+    dev->stats.pool_hits++;
+    dev->live.emplace(p, sz);
+    *ptr = p;
+    return POLAR_HIP_OK;
+  }
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, sz);
+  if (e == hipErrorOutOfMemory) {
+    // Give cached blocks back to the driver and try once more.  Work that
+    // still reads them may be in flight, so drain the stream first.
+    (void)hipGetLastError();
+    (void)hipStreamSynchronize(dev->stream);
+    dropCachedLocked(dev);
+    e = hipMalloc(&p, sz);
+  }
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    return failHip(e, "hipMalloc");
+  }
+  dev->stats.device_allocs++;
+  dev->stats.bytes_in_use += sz;
+  dev->live.emplace(p, sz);
+  *ptr = p;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_free(polar_hip_device* dev, void* ptr) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  if (ptr == nullptr) return POLAR_HIP_OK;
+  std::lock_guard<std::mutex> g(dev->mu);
+  auto it = dev->live.find(ptr);
+  if (it == dev->live.end())
+    return fail(POLAR_HIP_ERR_INVALID, "polar_hip_free: %p is not a live block",
+                ptr);
+  const uint64_t sz = it->second;
+  dev->live.erase(it);
+  dev->cached[sz].push_back(ptr);
+  dev->stats.bytes_in_use -= sz;
+  dev->stats.bytes_cached += sz;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_pool_trim(polar_hip_device* dev) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  std::lock_guard<std::mutex> g(dev->mu);
+  dropCachedLocked(dev);
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out) {
+  POLAR_HIP_REQUIRE(dev != nullptr && out != nullptr, "null argument");
+  std::lock_guard<std::mutex> g(dev->mu);
+  *out = dev->stats;
+  return POLAR_HIP_OK;
+}
+
+// ---- copies -----------------------------------------------------------------
+
+int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
+                             const void* src_host, uint64_t bytes) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  if (bytes == 0) return POLAR_HIP_OK;
+  POLAR_HIP_REQUIRE(dst_device != nullptr && src_host != nullptr,
+                    "null buffer");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipMemcpyAsync(dst_device, src_host, bytes,
+                               hipMemcpyHostToDevice, dev->stream));
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
+                           const void* src_device, uint64_t bytes) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  if (bytes == 0) return POLAR_HIP_OK;
+  POLAR_HIP_REQUIRE(dst_host != nullptr && src_device != nullptr,
+                    "null buffer");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes,
+                               hipMemcpyDeviceToHost, dev->stream));
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  return POLAR_HIP_OK;
+}
+
+// ---- events -----------------------------------------------------------------
+
+int polar_hip_event_record(polar_hip_device* dev, polar_hip_event** out) {
+  POLAR_HIP_REQUIRE(dev != nullptr && out != nullptr, "null argument");
+  *out = nullptr;
+  polar_hip_event* e = nullptr;
+  {
+    std::lock_guard<std::mutex> g(dev->mu);
+    if (!dev->idleEvents.empty()) {
+      e = dev->idleEvents.back();
+      dev->idleEvents.pop_back();
+    }
+  }
+  if (e == nullptr) {
+    POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+    hipEvent_t he;
+    POLAR_HIP_TRY(hipEventCreate(&he));
+    e = new polar_hip_event{dev, he};
+    std::lock_guard<std::mutex> g(dev->mu);
+    dev->allEvents.push_back(e);
+  }
+  hipError_t err = hipEventRecord(e->ev, dev->stream);
+  if (err != hipSuccess) {
+    std::lock_guard<std::mutex> g(dev->mu);
+    dev->idleEvents.push_back(e);
+    return failHip(err, "hipEventRecord");
+  }
+  *out = e;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_event_synchronize(polar_hip_event* evt) {
+  POLAR_HIP_REQUIRE(evt != nullptr, "evt is null");
+  POLAR_HIP_TRY(hipEventSynchronize(evt->ev));
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_event_query(polar_hip_event* evt, int* done) {
+  POLAR_HIP_REQUIRE(evt != nullptr && done != nullptr, "null argument");
+  hipError_t e = hipEventQuery(evt->ev);
+  if (e == hipSuccess) {
+    *done = 1;
+  } else if (e == hipErrorNotReady) {
+    (void)hipGetLastError();
+    *done = 0;
+  } else {
+    return failHip(e, "hipEventQuery");
+  }
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_stream_wait_event(polar_hip_device* dev, polar_hip_event* evt) {
+  POLAR_HIP_REQUIRE(dev != nullptr && evt != nullptr, "null argument");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipStreamWaitEvent(dev->stream, evt->ev, 0));
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_event_elapsed_ms(polar_hip_event* start, polar_hip_event* stop,
+                               float* ms) {
+  POLAR_HIP_REQUIRE(start && stop && ms, "null argument");
+  POLAR_HIP_TRY(hipEventElapsedTime(ms, start->ev, stop->ev));
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_event_release(polar_hip_event* evt) {
+  POLAR_HIP_REQUIRE(evt != nullptr, "evt is null");
+  std::lock_guard<std::mutex> g(evt->dev->mu);
+  evt->dev->idleEvents.push_back(evt);
+  return POLAR_HIP_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,128 @@
+"""Helpers shared by the parity tests: seeded input generators for the
+benchmark configurations, the tolerance rules, and a dispatcher that runs one
+golden-vector case on either the oracle or the device."""
+import json
+import os
+
+import numpy as np
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                      "reference_vectors.json")
+
+# Tolerances of the parity contract
+ELEMENTWISE_REL = 1e-5   # per element, relative
+MATMUL_FRO_REL = 1e-4    # relative Frobenius
+
+
+def golden_cases():
+    with open(GOLDEN) as fh:
+        return json.load(fh)
+
+
+def uniform(rng, n, lo, hi):
+    return (rng.random(n, dtype=np.float32) * np.float32(hi - lo) + np.float32(lo)).astype(np.float32)
+
+
+def normal(rng, shape, std=1.0):
+    return (rng.standard_normal(shape, dtype=np.float32) * np.float32(std)).astype(np.float32)
+
+
+def elementwise_rel_error(got, ref, scale=None):
+    """max |x-r| / max(|r|, 1e-5*scale): relative error with an absolute floor
+    where the reference value is ~0 (scale = largest magnitude involved)."""
+    got = np.asarray(got, dtype=np.float64).ravel()
+    ref = np.asarray(ref, dtype=np.float64).ravel()
+    if scale is None:
+        scale = float(np.max(np.abs(ref))) if ref.size else 1.0
+    floor = max(1e-5 * scale, 1e-30)
+    if got.size == 0:
+        return 0.0
+    return float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)))
+
+
+def frobenius_rel_error(got, ref):
+    got = np.asarray(got, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    den = np.linalg.norm(ref)
+    return float(np.linalg.norm(got - ref) / (den if den > 0 else 1.0))
+
+
+def stored_shapes(ta, tb, m, n, k):
+    return ((k, m) if ta else (m, k)), ((n, k) if tb else (k, n))
+
+
+def run_case_oracle(case):
+    import polar_oracle as o
+    kn = case["kernel"]
+    if kn == "fadd":
+        return o.fadd(case["a"], case["scaleA"], case["b"], case["scaleB"])
+    if kn == "fmul":
+        return o.fmul(case["a"], case["b"])
+    if kn == "fdivide":
+        return o.fdivide(case["a"], case["b"])
+    if kn == "fmulconcat":
+        return o.fmulconcat(case["gradient"], case["local"])
+    if kn == "fsigmoid":
+        return o.fsigmoid(case["x"])
+    if kn == "flogloss":
+        return o.flogloss(case["predicted"], case["truth"])
+    if kn == "fmatmul":
+        sa, sb = stored_shapes(case["transA"], case["transB"], case["m"], case["n"], case["k"])
+        a = np.asarray(case["a"], dtype=np.float32).reshape(sa)
+        b = np.asarray(case["b"], dtype=np.float32).reshape(sb)
+        return o.fmatmul(case["transA"], case["transB"], a, b).ravel()
+    raise KeyError(kn)
+
+
+def run_case_device(dev, case):
+    kn = case["kernel"]
+    bufs = []
+
+    def up(x):
+        b = dev.array(np.asarray(x, dtype=np.float32))
+        bufs.append(b)
+        return b
+    try:
+        if kn == "fadd":
+            a, b = up(case["a"]), up(case["b"])
+            c = dev.empty(a.count); bufs.append(c)
+            dev.fadd(a, case["scaleA"], b, case["scaleB"], c)
+        elif kn in ("fmul", "fdivide"):
+            a, b = up(case["a"]), up(case["b"])
+            c = dev.empty(a.count); bufs.append(c)
+            getattr(dev, kn)(a, b, c)
+        elif kn == "fmulconcat":
+            g, l = up(case["gradient"]), up(case["local"])
+            c = dev.empty(l.count); bufs.append(c)
+            dev.fmulconcat(g, l, c)
+        elif kn == "fsigmoid":
+            x = up(case["x"])
+            c = dev.empty(x.count); bufs.append(c)
+            dev.fsigmoid(x, c)
+        elif kn == "flogloss":
+            p, t = up(case["predicted"]), up(case["truth"])
+            c = dev.empty(p.count); bufs.append(c)
+            dev.flogloss(p, t, c)
+        elif kn == "fmatmul":
+            a, b = up(case["a"]), up(case["b"])
+            c = dev.empty(case["m"] * case["n"]); bufs.append(c)
+            dev.fmatmul(case["transA"], case["transB"], a, b, c, case["m"], case["n"], case["k"])
+        else:
+            raise KeyError(kn)
+        return c.download()
+    finally:
+        for b in bufs:
+            b.free()
+
+
+def check_case(case, got):
+    exp = np.asarray(case["expected"], dtype=np.float64)
+    got = np.asarray(got, dtype=np.float64).ravel()
+    assert got.shape == exp.shape
+    if case["exact"]:
+        assert np.array_equal(got.astype(np.float32), exp.astype(np.float32)), (case["cite"], got, exp)
+    else:
+        rel = np.abs(got - exp) / np.abs(exp)
+        assert np.all(rel <= case["rel_tol"]), (case["cite"], got, exp)
+        for i in case.get("exact_indices", []):
+            assert np.float32(got[i]) == np.float32(exp[i]), (case["cite"], i, got[i], exp[i])

@@ -1,0 +1,255 @@
+"""Parity of the gfx950 kernels with the CPU oracle, through the C ABI
+(include/polar_hip.h).  Bit-exact for the operations that are single IEEE
+operations or pure data movement; 1e-5 relative per element for
+sigmoid/logloss; 1e-4 relative Frobenius for matmul."""
+import numpy as np
+import pytest
+
+import parity
+import polar_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [1, 2, 3, 4, 5, 63, 64, 255, 256, 1023, 1024, 4099, 65536 + 7, 1000003]
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("case", parity.golden_cases(), ids=lambda c: c["kernel"] + "@" + c["cite"].split("/")[-1])
+def test_golden_vectors_on_device(dev, case):
+    _say("golden", case["cite"])
+    parity.check_case(case, parity.run_case_device(dev, case))
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("misalign", [0, 1])
+def test_binary_ops_bit_exact(dev, n, misalign):
+    _say("binary ops n=", n, "misalign=", misalign)
+    rng = np.random.default_rng(100 + n)
+    a = parity.uniform(rng, n, -1, 1)
+    b = parity.uniform(rng, n, -1, 1)
+    den = parity.uniform(rng, n, 0.5, 2)
+    da, db, dden = (dev.array(x, misalign) for x in (a, b, den))
+    dc = dev.empty(n, misalign)
+    dev.fadd(da, 1.0, db, 1.0, dc)
+    assert np.array_equal(dc.download(), o.fadd(a, 1.0, b, 1.0))
+    dev.fadd(da, 0.34, db, 0.21, dc)
+    assert np.array_equal(dc.download(), o.fadd(a, 0.34, b, 0.21))
+    dev.fmul(da, db, dc)
+    assert np.array_equal(dc.download(), o.fmul(a, b))
+    dev.fdivide(da, dden, dc)
+    assert np.array_equal(dc.download(), o.fdivide(a, den))
+    for x in (da, db, dden, dc):
+        x.free()
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_mixed_alignment(dev, n):
+    # one operand 16-byte aligned, the other not: must take the dword path
+    _say("mixed alignment n=", n)
+    rng = np.random.default_rng(200 + n)
+    a, b = parity.uniform(rng, n, -1, 1), parity.uniform(rng, n, -1, 1)
+    da, db, dc = dev.array(a, 0), dev.array(b, 3), dev.empty(n, 2)
+    dev.fmul(da, db, dc)
+    assert np.array_equal(dc.download(), o.fmul(a, b))
+    for x in (da, db, dc):
+        x.free()
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("misalign", [0, 1])
+def test_unary_and_fill(dev, n, misalign):
+    _say("unary n=", n, "misalign=", misalign)
+    rng = np.random.default_rng(300 + n)
+    x = parity.uniform(rng, n, -1, 1)
+    g = np.array([np.float32(-2.5), 9.0], dtype=np.float32)
+    dx, dg, dout = dev.array(x, misalign), dev.array(g), dev.empty(n, misalign)
+    dev.fcopy(dx, dout)
+    assert np.array_equal(dout.download(), x)
+    dev.ffill(3.0, dout)
+    assert np.array_equal(dout.download(), o.ffill(3.0, n))
+    dev.fmulconcat(dg, dx, dout)
+    assert np.array_equal(dout.download(), o.fmulconcat(g, x))
+    for b in (dx, dg, dout):
+        b.free()
+
+
+@pytest.mark.parametrize("n", SIZES)
+def test_sigmoid_logloss(dev, n):
+    _say("sigmoid/logloss n=", n)
+    rng = np.random.default_rng(400 + n)
+    x = parity.uniform(rng, n, -1, 1)
+    wide = parity.uniform(rng, n, -30, 30)  # reaches both clamps
+    y = (rng.random(n) < 0.1).astype(np.float32)
+    dx, dw, dy, dp, dl = dev.array(x), dev.array(wide), dev.array(y), dev.empty(n), dev.empty(n)
+    dev.fsigmoid(dx, dp)
+    p = dp.download()
+    assert parity.elementwise_rel_error(p, o.fsigmoid(x)) <= parity.ELEMENTWISE_REL
+    dev.flogloss(dp, dy, dl)
+    assert parity.elementwise_rel_error(dl.download(), o.flogloss(p, y)) <= parity.ELEMENTWISE_REL
+    dev.fsigmoid(dw, dp)
+    pw = dp.download()
+    ref = o.fsigmoid(wide)
+    assert parity.elementwise_rel_error(pw, ref) <= parity.ELEMENTWISE_REL
+    eps = np.float32(1e-5)
+    assert pw.min() >= eps and pw.max() <= np.float32(1) - eps
+    dev.flogloss(dp, dy, dl)
+    assert parity.elementwise_rel_error(dl.download(), o.flogloss(pw, y)) <= parity.ELEMENTWISE_REL
+    for b in (dx, dw, dy, dp, dl):
+        b.free()
+
+
+def test_sigmoid_special_values(dev):
+    xs = np.array([0.0, -100.0, 100.0, -200.0, 1e30, -1e30, -11.0, 11.0, -12.0, 12.0], dtype=np.float32)
+    dx, dp = dev.array(xs), dev.empty(xs.size)
+    dev.fsigmoid(dx, dp)
+    got, ref = dp.download(), o.fsigmoid(xs)
+    assert parity.elementwise_rel_error(got, ref) <= parity.ELEMENTWISE_REL
+    eps = np.float32(1e-5)
+    assert got[0] == np.float32(0.5)
+    assert got[1] == eps and got[3] == eps and got[5] == eps and got[8] == eps
+    assert got[2] == np.float32(1) - eps and got[4] == np.float32(1) - eps and got[9] == np.float32(1) - eps
+    dx.free(); dp.free()
+
+
+def test_empty_inputs(dev):
+    a = dev.empty(4)
+    for fn in (lambda: dev.fadd(a, 1.0, a, 1.0, a, 0), lambda: dev.fmul(a, a, a, 0),
+               lambda: dev.fsigmoid(a, a, 0), lambda: dev.ffill(1.0, a, 0),
+               lambda: dev.ftranspose(a, a, 0, 5), lambda: dev.fmatmul(0, 0, a, a, a, 0, 4, 4)):
+        fn()
+    dev.synchronize()
+    a.free()
+
+
+def test_in_place_update(dev):
+    # the framework's weight update writes fadd's result into its first operand
+    rng = np.random.default_rng(9)
+    w, g = parity.normal(rng, 100003), parity.normal(rng, 100003)
+    dw, dg = dev.array(w), dev.array(g)
+    dev.fadd(dw, 1.0, dg, -0.01, dw)
+    assert np.array_equal(dw.download(), o.fadd(w, 1.0, g, -0.01))
+    dw.free(); dg.free()
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (1, 7), (7, 1), (3, 5), (64, 64), (65, 63), (64, 1000),
+                                   (1000, 64), (257, 129), (1031, 517)])
+def test_transpose(dev, shape):
+    _say("transpose", shape)
+    rng = np.random.default_rng(shape[0] * 7919 + shape[1])
+    x = parity.normal(rng, shape)
+    dx, dt, dtt = dev.array(x), dev.empty(x.size), dev.empty(x.size)
+    dev.ftranspose(dx, dt, shape[0], shape[1])
+    assert np.array_equal(dt.download((shape[1], shape[0])), o.ftranspose(x))
+    dev.ftranspose(dt, dtt, shape[1], shape[0])  # involution
+    assert np.array_equal(dtt.download(shape), x)
+    for b in (dx, dt, dtt):
+        b.free()
+
+
+MM_SHAPES = [(1, 1, 4), (2, 2, 2), (2, 3, 4), (1, 1, 1), (5, 7, 3), (32, 32, 32), (64, 64, 64),
+             (128, 128, 128), (256, 384, 512), (130, 70, 50), (127, 33, 65), (33, 127, 129),
+             (200, 10, 784), (256, 10, 784), (129, 257, 1), (300, 300, 300), (512, 512, 2048)]
+
+
+def _matmul_device(dev, ta, tb, a, b, m, n, k, misalign=0):
+    da, db, dc = dev.array(a, misalign), dev.array(b, misalign), dev.empty(m * n, misalign)
+    dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+    out = dc.download((m, n))
+    for x in (da, db, dc):
+        x.free()
+    return out
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("mnk", MM_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul(dev, ta, tb, mnk):
+    m, n, k = mnk
+    _say("matmul", ta, tb, mnk)
+    rng = np.random.default_rng(m * 1000003 + n * 1009 + k + 2 * ta + tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+    got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+    ref = o.fmatmul(ta, tb, a, b)
+    assert parity.frobenius_rel_error(got, ref) <= parity.MATMUL_FRO_REL
+    # no element is left unwritten or badly off either
+    assert np.max(np.abs(got - ref)) <= 1e-3 * max(1.0, np.sqrt(k))
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_integer_exact_and_tt_identity(dev, ta, tb):
+    # small integers: every partial sum is exact in fp32 whatever the order
+    rng = np.random.default_rng(11 + 2 * ta + tb)
+    m, n, k = 150, 90, 210
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a = rng.integers(-8, 9, sa).astype(np.float32)
+    b = rng.integers(-8, 9, sb).astype(np.float32)
+    got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+    assert np.array_equal(got, o.fmatmul(ta, tb, a, b))
+    if ta and tb:  # (A^T B^T) = (B A)^T
+        ba = _matmul_device(dev, False, False, b, a, n, m, k)
+        assert np.array_equal(got, ba.T)
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_unaligned_base(dev, ta, tb):
+    rng = np.random.default_rng(21 + 2 * ta + tb)
+    m, n, k = 132, 68, 100
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+    got = _matmul_device(dev, ta, tb, a, b, m, n, k, misalign=1)
+    assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+
+
+def test_matmul_overwrites_output(dev):
+    # no beta: C is overwritten, stale contents must not leak
+    rng = np.random.default_rng(31)
+    a, b = parity.normal(rng, (70, 40)), parity.normal(rng, (40, 50))
+    da, db, dc = dev.array(a), dev.array(b), dev.array(np.full(70 * 50, 1e9, dtype=np.float32))
+    dev.fmatmul(False, False, da, db, dc, 70, 50, 40)
+    assert parity.frobenius_rel_error(dc.download((70, 50)), o.fmatmul(False, False, a, b)) <= parity.MATMUL_FRO_REL
+    for x in (da, db, dc):
+        x.free()
+
+
+def test_transpose_matmul_cross_identity(dev):
+    # matmul_t_f(A, B) == matmul_f_f(T(A), B) with integer data (exact)
+    rng = np.random.default_rng(41)
+    k, m, n = 77, 130, 45
+    a = rng.integers(-8, 9, (k, m)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    da, db, dat, c1, c2 = dev.array(a), dev.array(b), dev.empty(a.size), dev.empty(m * n), dev.empty(m * n)
+    dev.ftranspose(da, dat, k, m)
+    dev.fmatmul(True, False, da, db, c1, m, n, k)
+    dev.fmatmul(False, False, dat, db, c2, m, n, k)
+    assert np.array_equal(c1.download(), c2.download())
+    for x in (da, db, dat, c1, c2):
+        x.free()
+
+
+def test_pool_reuses_blocks(dev):
+    dev.synchronize()
+    s0 = dev.pool_stats()
+    b = dev.empty(1 << 20)
+    b.free()
+    c = dev.empty(1 << 20)
+    s1 = dev.pool_stats()
+    c.free()
+    assert s1.pool_hits >= s0.pool_hits + 1
+    assert s1.device_allocs <= s0.device_allocs + 1
+
+
+def test_events_order_and_time(dev):
+    x = dev.empty(1 << 22)
+    e0 = dev.record()
+    dev.ffill(1.0, x)
+    e1 = dev.record()
+    e1.synchronize()
+    assert e0.done() and e1.done()
+    assert e0.elapsed_ms(e1) > 0
+    e0.release(); e1.release(); x.free()
