@@ -1,0 +1,291 @@
+#!/usr/bin/env python3
+"""Benchmark of the builtin-operation kernels on one MI355X.
+
+One "step" is one pass of the elementwise bandwidth sweep: fadd, fmul,
+fdivide, fsigmoid, fcopy and ffill(3.0), each as a single kernel over fp32
+tensors of 2^26 elements that are already resident in HBM.  `value` is the
+algorithmic bytes of the whole sweep divided by the wall time of the timed
+steps.  After the timed region the same run measures ftranspose 12345x6789,
+the 4096^3 fp32 matmul in all four transpose variants, and the CPU oracle on
+the host cores (a reported baseline only).
+
+Per-kernel durations come from HIP events recorded on the library's own
+stream around every launch inside the timed region.
+
+Prints ONE JSON line on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_FP32_PEAK_TFLOPS = 157.3  # MI355X dense fp32 matrix, published
+
+N_SWEEP = 1 << 26
+# algorithmic bytes per element (reads + writes, fp32, scalars free)
+BYTES_PER_ELEMENT = {"fadd": 12, "fmul": 12, "fdivide": 12, "fsigmoid": 8,
+                     "fcopy": 8, "ffill": 4, "flogloss": 12, "fmulconcat": 8,
+                     "ftranspose": 8}
+SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
+T_ROWS, T_COLS = 12345, 6789
+MM = 4096
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_inputs(n):
+    rng = np.random.default_rng(20240607)
+    a = (rng.random(n, dtype=np.float32) * 2 - 1).astype(np.float32)      # U[-1,1)
+    b = (rng.random(n, dtype=np.float32) * 2 - 1).astype(np.float32)      # U[-1,1)
+    den = (rng.random(n, dtype=np.float32) * 1.5 + 0.5).astype(np.float32)  # U[0.5,2)
+    return a, b, den
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--elements", type=int, default=N_SWEEP,
+                    help="elements per tensor in the sweep (default 2^26)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-matmul", action="store_true", help="skip the matmul/transpose legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this runtime drives one GPU; --gpus must be 1 "
+                 "(no multi-GPU path exists in this build)")
+
+    import __graft_entry__ as entry
+    entry.load_package()
+    from polarai_framework_amd import capi
+
+    n = args.elements
+    dev = capi.Device(0)
+    info = dev.info()
+    log(f"device: {info.name.decode()} {info.arch.decode()} CUs={info.compute_units} "
+        f"clock={info.clock_khz / 1e6:.2f} GHz memclk={info.memory_clock_khz / 1e6:.2f} GHz "
+        f"bus={info.memory_bus_bits} bit")
+
+    a, b, den = make_inputs(n)
+    da, db, dden = dev.array(a), dev.array(b), dev.array(den)
+    outs = {op: dev.empty(n) for op in SWEEP}
+
+    def launch(op):
+        if op == "fadd":
+            dev.fadd(da, 1.0, db, 1.0, outs[op])
+        elif op == "fmul":
+            dev.fmul(da, db, outs[op])
+        elif op == "fdivide":
+            dev.fdivide(da, dden, outs[op])
+        elif op == "fsigmoid":
+            dev.fsigmoid(da, outs[op])
+        elif op == "fcopy":
+            dev.fcopy(da, outs[op])
+        elif op == "ffill":
+            dev.ffill(3.0, outs[op])
+
+    def step(events=None):
+        for op in SWEEP:
+            if events is not None:
+                events.append(dev.record())
+            launch(op)
+        if events is not None:
+            events.append(dev.record())
+
+    for _ in range(args.warmup):
+        step()
+    dev.synchronize()
+    all_events = []
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ev = []
+        step(ev)
+        all_events.append(ev)
+    dev.synchronize()
+    t1 = time.perf_counter()
+    wall = t1 - t0
+
+    per_op_ms = {op: [] for op in SWEEP}
+    for ev in all_events:
+        for i, op in enumerate(SWEEP):
+            per_op_ms[op].append(ev[i].elapsed_ms(ev[i + 1]))
+        for e in ev:
+            e.release()
+    step_bytes = sum(BYTES_PER_ELEMENT[op] * n for op in SWEEP)
+    value = step_bytes * args.steps / wall / 1e9
+
+    per_op = {}
+    for op in SWEEP:
+        ms = float(np.mean(per_op_ms[op]))
+        gbs = BYTES_PER_ELEMENT[op] * n / (ms * 1e-3) / 1e9
+        per_op[op] = {"ms": round(ms, 5), "min_ms": round(float(np.min(per_op_ms[op])), 5),
+                      "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        log(f"{op:10s} {ms * 1e3:9.1f} us  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of HBM peak")
+    dominant = max(SWEEP, key=lambda op: np.mean(per_op_ms[op]))
+    roofline = {"bound": "hbm", "kernel": dominant,
+                "achieved": per_op[dominant]["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(per_op[dominant]["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None}
+
+    # quick sanity of what was timed (full parity lives in tests/)
+    probe = outs["fadd"].download()[:1024]
+    assert np.array_equal(probe, (a[:1024] + b[:1024]).astype(np.float32)), "fadd output is wrong"
+
+    result = {
+        "metric": "elementwise GB/s + fp32 matmul GFLOP/s, % of MI355X roofline, 1 GPU",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "elementwise bandwidth sweep: fadd fmul fdivide fsigmoid fcopy "
+                               f"ffill(3.0), fp32, {n} elements per tensor, one kernel each",
+                   "elements": n, "bytes_per_step": step_bytes},
+        "device": {"name": info.name.decode(), "arch": info.arch.decode(),
+                   "compute_units": info.compute_units, "clock_khz": info.clock_khz,
+                   "memory_clock_khz": info.memory_clock_khz, "memory_bus_bits": info.memory_bus_bits},
+        "roofline": roofline,
+        "per_op": per_op,
+    }
+
+    for buf in list(outs.values()) + [dden]:
+        buf.free()
+
+    if not args.no_matmul:
+        result["transpose"] = bench_transpose(dev, args)
+        result["matmul"] = bench_matmul(dev, args)
+    da.free(); db.free()
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(a, b, den, n)
+
+    dev.close()
+    print(json.dumps(result), flush=True)
+
+
+def time_kernel(dev, fn, warmup, reps):
+    for _ in range(warmup):
+        fn()
+    dev.synchronize()
+    ms = []
+    for _ in range(reps):
+        e0 = dev.record()
+        fn()
+        e1 = dev.record()
+        e1.synchronize()
+        ms.append(e0.elapsed_ms(e1))
+        e0.release(); e1.release()
+    return ms
+
+
+def bench_transpose(dev, args):
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((T_ROWS, T_COLS), dtype=np.float32)
+    dx, dt = dev.array(x), dev.empty(x.size)
+    ms = time_kernel(dev, lambda: dev.ftranspose(dx, dt, T_ROWS, T_COLS), args.warmup, args.steps)
+    got = dt.download((T_COLS, T_ROWS))
+    assert np.array_equal(got[:64], x.T[:64]), "transpose output is wrong"
+    dx.free(); dt.free()
+    nbytes = 8 * T_ROWS * T_COLS
+    gbs = nbytes / (np.mean(ms) * 1e-3) / 1e9
+    log(f"ftranspose {np.mean(ms) * 1e3:9.1f} us  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of HBM peak")
+    return {"workload": f"ftranspose {T_ROWS}x{T_COLS} fp32", "ms": round(float(np.mean(ms)), 5),
+            "min_ms": round(float(np.min(ms)), 5), "GB/s": round(gbs, 1),
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+
+
+def bench_matmul(dev, args):
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal((MM, MM), dtype=np.float32)
+    b = rng.standard_normal((MM, MM), dtype=np.float32)
+    da, db, dc = dev.array(a), dev.array(b), dev.empty(MM * MM)
+    flops = 2.0 * MM ** 3
+    out = {"workload": f"fmatmul {MM}x{MM}x{MM} fp32 N(0,1), C overwritten", "variants": {}}
+    worst = None
+    for ta in (0, 1):
+        for tb in (0, 1):
+            name = f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'}"
+            ms = time_kernel(dev, lambda: dev.fmatmul(ta, tb, da, db, dc, MM, MM, MM),
+                             max(1, args.warmup), max(5, args.steps))
+            tf = flops / (np.mean(ms) * 1e-3) / 1e12
+            # spot check: 4 rows against an fp64 product
+            got = dc.download((MM, MM))[:4]
+            A = a.T if ta else a
+            B = b.T if tb else b
+            ref = A[:4].astype(np.float64) @ B.astype(np.float64)
+            err = np.linalg.norm(got - ref) / np.linalg.norm(ref)
+            assert err < 1e-4, (name, err)
+            out["variants"][name] = {"ms": round(float(np.mean(ms)), 5), "min_ms": round(float(np.min(ms)), 5),
+                                     "GFLOP/s": round(tf * 1e3, 1),
+                                     "frac_mfma_fp32_peak": round(tf / MFMA_FP32_PEAK_TFLOPS, 4)}
+            log(f"{name} {np.mean(ms):8.3f} ms  {tf:7.2f} TFLOP/s  {100 * tf / MFMA_FP32_PEAK_TFLOPS:5.1f}% of fp32 MFMA peak")
+            if worst is None or tf < worst:
+                worst = tf
+    for x in (da, db, dc):
+        x.free()
+    mean_tf = float(np.mean([v["GFLOP/s"] for v in out["variants"].values()])) / 1e3
+    out["GFLOP/s"] = round(mean_tf * 1e3, 1)
+    out["roofline"] = {"bound": "mfma", "achieved": round(mean_tf, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
+                       "unit": "TFLOP/s", "frac": round(mean_tf / MFMA_FP32_PEAK_TFLOPS, 4),
+                       "worst_variant_frac": round(worst / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None}
+    return out
+
+
+def cpu_baseline(a, b, den, n):
+    """The CPU oracle (a restatement of the reference's host kernels; the
+    reference's own host runtime cannot be built here) timed on this box's
+    host cores on the same inputs: one full sweep with all cores, one with a
+    single thread, and a 1024^3 matmul with a single thread."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import polar_oracle as o
+    cores = o.hw_threads()
+    lib = o.lib()
+    out = np.empty(n, dtype=np.float32)
+
+    def sweep():
+        lib.polar_oracle_fadd(a, 1.0, b, 1.0, out, n)
+        lib.polar_oracle_fmul(a, b, out, n)
+        lib.polar_oracle_fdivide(a, den, out, n)
+        lib.polar_oracle_fsigmoid(a, out, n)
+        lib.polar_oracle_fcopy(a, out, n)
+        lib.polar_oracle_ffill(3.0, out, n)
+
+    step_bytes = sum(BYTES_PER_ELEMENT[op] * n for op in SWEEP)
+    res = {}
+    for threads in (cores, 1):
+        o.set_threads(threads)
+        sweep()  # warm-up (page faults of `out`)
+        reps = 3 if threads > 1 else 1
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            sweep()
+        dt = (time.perf_counter() - t0) / reps
+        res[threads] = step_bytes / dt / 1e9
+        log(f"cpu oracle sweep, {threads} thread(s): {dt * 1e3:.1f} ms/step, {res[threads]:.2f} GB/s")
+    o.set_threads(1)
+    k = 1024
+    rng = np.random.default_rng(8)
+    ma = rng.standard_normal((k, k), dtype=np.float32)
+    mb = rng.standard_normal((k, k), dtype=np.float32)
+    t0 = time.perf_counter()
+    o.fmatmul(False, False, ma, mb)
+    mm_dt = time.perf_counter() - t0
+    log(f"cpu oracle fmatmul_f_f 1024^3, 1 thread: {mm_dt:.2f} s, {2 * k ** 3 / mm_dt / 1e9:.2f} GFLOP/s")
+    return {"value": round(res[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"the full sweep ({n} elements per tensor, same inputs), {cores} host threads, "
+                      "mean of 3 passes after one warm-up pass",
+            "single_thread_value": round(res[1], 2),
+            "matmul_1024_single_thread_GFLOP/s": round(2 * k ** 3 / mm_dt / 1e9, 3)}
+
+
+if __name__ == "__main__":
+    main()
