@@ -1,0 +1,101 @@
+// The seven C symbols that JIT-compiled graph code calls
+// (src/backend/generic/runtime/support/api.hpp:15-32, bodies in
+// src/backend/generic/runtime/support/routines.cpp:24-102; LLVM prototypes in
+// utils/dialects/lib/Passes/DeployDefaultFunctions.cpp:38-108), restated for
+// the mini-executor.  "host" nodes go to the RAM side of the allocator, every
+// other device to its own layer.
+#include "support_routines.hpp"
+
+#include <cstring>
+
+using namespace polar_harness_detail;
+
+namespace {
+// src/backend/generic/runtime/utils/utils.hpp:7-17
+MemoryRecord toRecord(const TensorInfo* t) {
+  size_t bytes;
+  switch (static_cast<polarai::core::DataType>(t->dataType)) {
+  case polarai::core::DataType::DOUBLE: bytes = 8; break;
+  case polarai::core::DataType::FLOAT: bytes = 4; break;
+  case polarai::core::DataType::HALF: bytes = 2; break;
+  default: fatalError(kFatalOther, "Size for dataType is not defined");
+  }
+  for (uint64_t i = 0; i < t->dims; ++i) bytes *= t->shape[i];
+  return MemoryRecord{static_cast<size_t>(t->virtAddr), bytes};
+}
+bool isHost(Device& d) { return d.getDeviceName() == "host"; }
+} // namespace
+
+namespace polar_harness_detail {
+uint64_t g_deferredReleases = 0;
+uint64_t g_eventsWaited = 0;
+} // namespace polar_harness_detail
+
+extern "C" {
+
+void ath_allocate(GraphHandle* handle, Device& device, TensorInfo* tensor) {
+  const MemoryRecord rec = toRecord(tensor);
+  if (isHost(device))
+    handle->allocator->allocate(rec);
+  else
+    handle->allocator->allocate(rec, device);
+}
+
+// With an event the release is deferred to the event's callbacks, which run
+// when somebody waits on it (the barrier).
+void ath_release(GraphHandle* handle, Device& device, TensorInfo* tensor, Event* blockingEvt) {
+  const MemoryRecord rec = toRecord(tensor);
+  if (isHost(device)) {
+    handle->allocator->release(rec);
+  } else if (blockingEvt != nullptr) {
+    Device* dev = &device;
+    blockingEvt->addCallback([handle, dev, rec]() {
+      ++g_deferredReleases;
+      handle->allocator->release(rec, *dev);
+    });
+  } else {
+    handle->allocator->release(rec, device);
+  }
+}
+
+void ath_lock(GraphHandle* handle, Device& device, TensorInfo* tensor, LockType type) {
+  const MemoryRecord rec = toRecord(tensor);
+  if (isHost(device))
+    handle->allocator->lock(rec, type);
+  else
+    handle->allocator->lock(rec, device, type);
+}
+
+Device* ath_device_select(GraphHandle* handle, uint64_t nodeId) {
+  if (handle->isHostNode.count(nodeId)) return handle->devices.back().get();
+  return handle->devices.front().get();
+}
+
+void ath_barrier(uint32_t count, Event** events) {
+  for (uint32_t i = 0; i < count; ++i) {
+    if (events[i] != nullptr) {
+      ++g_eventsWaited;
+      events[i]->wait();
+    }
+  }
+}
+
+Event* ath_launch(GraphHandle* handle, Device* device, Event* event, LaunchCommand& command) {
+  return device->launch(*handle->allocator, command, event);
+}
+
+void ath_load(GraphHandle* handle, uint64_t nodeId, TensorInfo* tensor) {
+  auto it = handle->mLoaders.find(nodeId);
+  if (it == handle->mLoaders.end() || it->second == nullptr)
+    fatalError(kFatalOther, "No loader for node %llu", static_cast<unsigned long long>(nodeId));
+  const MemoryRecord rec = toRecord(tensor);
+  void* ptr = handle->allocator->get(rec);
+  const auto type = static_cast<polarai::core::DataType>(tensor->dataType);
+  if (type == polarai::core::DataType::FLOAT) {
+    it->second->load(static_cast<float*>(ptr), rec.allocationSize / 4);
+  } else if (type == polarai::core::DataType::DOUBLE) {
+    fatalError(kFatalOther, "Double is not supported.");
+  }
+}
+
+} // extern "C"

@@ -1,0 +1,152 @@
+// Classes of the MI355X runtime plugin (libpolar_rt_hip.so): the Context,
+// Device, Event and allocator layer the framework's runtime driver receives
+// from initContext().  They sit on the C ABI of the device library
+// (polar_hip.h); no HIP header is needed here.
+//
+// Built with -fno-rtti -fno-exceptions like the framework's core
+// (CMakeModules/PolarTarget.cmake:8-13): nothing throws across the boundary and
+// no dynamic_cast is applied to objects that come from the caller.  Failures
+// follow the framework's convention for runtimes -- print and terminate
+// (src/backend/generic/runtime/hip/HIPContext.cpp:23-33,
+//  src/backend/generic/runtime/cuda/utils.hpp:20-28).
+#pragma once
+
+#include "polar_hip.h"
+#include "polar_rt_abi.hpp"
+
+#include <deque>
+#include <mutex>
+
+namespace polarai::backend::generic::mi355x {
+
+[[noreturn]] void fatal(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void checkStatus(int status, const char* what);
+
+// Device-memory layer of one GPU.  Takes the place of the per-tensor raw
+// allocations of the framework's allocator layers
+// (src/backend/generic/runtime/cuda/CudaAllocator.hpp:26-91,
+//  src/backend/generic/runtime/sycl/USMAllocator.h:30-107): records are keyed
+// by virtual address, memory comes from the device library's pool, and the
+// out-of-memory hook is live -- released records are handed to the registered
+// offload callback and then evicted.
+class HipPoolAllocator final : public AllocatorLayerBase {
+public:
+  explicit HipPoolAllocator(polar_hip_device* dev) : mDev(dev) {}
+  ~HipPoolAllocator() override;
+
+  void registerMemoryOffloadCallback(MemoryOffloadCallbackT cb) override;
+  void allocate(MemoryRecord record) override;
+  void deallocate(MemoryRecord record) override;
+  void lock(MemoryRecord record) override;
+  void release(MemoryRecord record) override;
+  void* getPtr(MemoryRecord record) override;
+  bool isAllocated(const MemoryRecord& record) const override;
+  size_t getTag(MemoryRecord record) override;
+  void setTag(MemoryRecord record, size_t tag) override;
+
+  // not part of the interface: capacity limit for tests of the eviction path
+  void setByteLimit(uint64_t bytes) { mByteLimit = bytes; }
+  // called by the owning device just before it closes: frees every block and
+  // turns the layer into an empty shell for owners that outlive the device
+  void detach();
+  uint64_t bytesHeld() const { return mBytesHeld; }
+
+private:
+  struct Entry {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+    size_t tag = 0;
+    bool locked = false;
+    bool released = false;
+  };
+  bool evictOneLocked(std::unique_lock<std::mutex>& guard);
+
+  polar_hip_device* mDev;
+  mutable std::mutex mMutex;
+  std::unordered_map<size_t, Entry> mEntries; // by virtual address
+  MemoryOffloadCallbackT mOffload;
+  uint64_t mByteLimit = 0; // 0 = limited by the device only
+  uint64_t mBytesHeld = 0;
+};
+
+class HipDevice;
+
+// One point in the stream order of a device.  wait() blocks until the stream
+// has reached it and then runs the callbacks on the calling thread, as the
+// framework's events do (src/backend/generic/runtime/cuda/CudaEvent.cpp:21-29).
+class HipEvent final : public Event {
+public:
+  HipEvent(HipDevice* device, polar_hip_event* native)
+      : mDevice(device), mNative(native) {}
+  ~HipEvent() override;
+  void wait() override;
+  void addCallback(std::function<void()> cb) override;
+  auto getDevice() -> Device* override;
+
+  void rearm(polar_hip_event* native);
+  bool idle();
+
+private:
+  HipDevice* mDevice;
+  polar_hip_event* mNative; // null once the stream is known to have passed it
+  std::mutex mMutex;
+  std::vector<std::function<void()>> mCallbacks;
+};
+
+class HipDevice final : public Device {
+public:
+  HipDevice(int ordinal);
+  ~HipDevice() override;
+
+  DeviceProvider getProvider() const override { return DeviceProvider::HIP; }
+  DeviceKind getKind() const override { return DeviceKind::GPU; }
+  std::string getDeviceName() const override { return mName; }
+  bool isPartitionSupported(PartitionDomain) override { return false; }
+  bool hasAllocator() override { return true; }
+  std::vector<std::shared_ptr<Device>> partition(PartitionDomain) override {
+    return {};
+  }
+  std::shared_ptr<AllocatorLayerBase> getAllocator() override {
+    return mAllocator;
+  }
+  bool operator==(const Device& other) const override {
+    return other.getDeviceName() == mName;
+  }
+  void copyToHost(MemoryRecord record, void* dest) const override;
+  void copyToDevice(MemoryRecord record, void* src) const override;
+  Event* launch(BackendAllocator& allocator, LaunchCommand& cmd,
+                Event* blockingEvent) override;
+  void consumeEvent(Event* evt) override;
+  void selectBinary(std::vector<std::shared_ptr<ProgramDesc>>&) override {}
+
+  polar_hip_device* native() const { return mDev; }
+  float* resolve(BackendAllocator& allocator, const MemoryRecord& record);
+
+private:
+  HipEvent* newEvent();
+
+  polar_hip_device* mDev = nullptr;
+  std::string mName;
+  std::shared_ptr<HipPoolAllocator> mAllocator;
+  std::mutex mEventMutex;
+  std::deque<std::unique_ptr<HipEvent>> mEvents; // every event ever returned
+  std::vector<HipEvent*> mIdleEvents;            // handed back via consumeEvent
+};
+
+class HipContext final : public Context {
+public:
+  HipContext();
+  ~HipContext() override = default;
+  std::vector<std::shared_ptr<Device>>& getDevices() override {
+    return mDevices;
+  }
+
+private:
+  std::vector<std::shared_ptr<Device>> mDevices;
+};
+
+// nativeKernelName -> launcher.  Returns false for an unknown name.
+bool dispatchNativeKernel(HipDevice& device, BackendAllocator& allocator,
+                          LaunchCommand& cmd);
+
+} // namespace polarai::backend::generic::mi355x

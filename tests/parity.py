@@ -126,3 +126,56 @@ def check_case(case, got):
         assert np.all(rel <= case["rel_tol"]), (case["cite"], got, exp)
         for i in case.get("exact_indices", []):
             assert np.float32(got[i]) == np.float32(exp[i]), (case["cite"], i, got[i], exp[i])
+
+
+# ---- per-node checking of a kernel DAG run through the mini-executor ---------
+
+BIT_EXACT_KERNELS = {"fadd", "fmul", "fdivide", "fmulconcat", "fcopy", "ffill", "ftranspose"}
+
+
+def oracle_node(node, values):
+    """Oracle result of one compute node of polarai_framework_amd.graphs, fed
+    with the operand values the device consumed (`values`: tensor key ->
+    array)."""
+    import polar_oracle as o
+    ins = [values[a.tensor_key] if hasattr(a, "tensor_key") else a for a in node.args[:-1]]
+    k = node.kernel
+    if k == "fadd":
+        return o.fadd(ins[0], ins[1], ins[2], ins[3])
+    if k == "fmul":
+        return o.fmul(ins[0], ins[1])
+    if k == "fdivide":
+        return o.fdivide(ins[0], ins[1])
+    if k == "fsigmoid":
+        return o.fsigmoid(ins[0])
+    if k == "flogloss":
+        return o.flogloss(ins[0], ins[1])
+    if k == "fmulconcat":
+        return o.fmulconcat(ins[0], ins[1])
+    if k.startswith("fmatmul_"):
+        return o.fmatmul(k[8] == "t", k[10] == "t", ins[0], ins[1])
+    raise KeyError(k)
+
+
+def check_graph_nodes(graph, values):
+    """Every compute node of `graph`: device output (values[result]) against
+    the oracle on the same operands.  Returns {node name: error}."""
+    report = {}
+    for node in graph.nodes:
+        if node.kind != "op":
+            continue
+        got = values[node.tensor_key]
+        ref = oracle_node(node, values).reshape(got.shape)
+        label = f"{graph.name}:{node.name or node.kernel}"
+        if node.kernel in BIT_EXACT_KERNELS:
+            assert np.array_equal(got, ref), label
+            report[label] = 0.0
+        elif node.kernel.startswith("fmatmul"):
+            err = frobenius_rel_error(got, ref)
+            assert err <= MATMUL_FRO_REL, (label, err)
+            report[label] = err
+        else:
+            err = elementwise_rel_error(got, ref)
+            assert err <= ELEMENTWISE_REL, (label, err)
+            report[label] = err
+    return report

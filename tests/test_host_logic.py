@@ -1,0 +1,170 @@
+"""CPU tests of the host side: the libraries load and export what the headers
+declare, the coherence protocol and call sequence of the mini-executor (on its
+mock device), and the failure conventions.  No compute is called: there is no
+GPU here."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from polarai_framework_amd import LIB_DEVICE, LIB_HARNESS, LIB_PLUGIN, REPO_ROOT, capi, harness
+
+
+def _declared(header, prefix):
+    text = open(os.path.join(REPO_ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(" + prefix + r"\w+)\s*\(", text)))
+
+
+def test_device_library_exports_every_declared_symbol():
+    names = _declared("polar_hip.h", "polar_hip_")
+    assert len(names) >= 29
+    lib = C.CDLL(LIB_DEVICE)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(capi.SIGNATURES) == names  # the binding covers the header exactly
+
+
+def test_harness_library_exports_every_declared_symbol():
+    names = _declared("polar_harness.h", "polar_harness_")
+    lib = C.CDLL(LIB_HARNESS)
+    for n in names:
+        assert hasattr(lib, n), n
+    assert sorted(harness.SIGNATURES) == names
+    for n in ("ath_allocate", "ath_release", "ath_lock", "ath_device_select", "ath_barrier",
+              "ath_launch", "ath_load"):
+        assert hasattr(lib, n), n
+
+
+def test_plugin_exports_driver_entry_points():
+    # what the runtime driver resolves: src/backend/generic/runtime/driver/RuntimeDriver.cpp:28-31
+    assert os.path.basename(LIB_PLUGIN) == "libpolar_rt_hip.so"
+    lib = C.CDLL(LIB_PLUGIN, mode=os.RTLD_LAZY | os.RTLD_LOCAL)
+    assert hasattr(lib, "initContext") and hasattr(lib, "closeContext")
+
+
+def test_device_library_without_gpu_reports_no_device():
+    if capi.device_count() != 0:
+        pytest.skip("a GPU is present")
+    with pytest.raises(capi.PolarHipError) as e:
+        capi.Device(0)
+    assert e.value.status == 2
+
+
+def test_null_arguments_are_rejected_not_dereferenced():
+    lib = capi.load_library()
+    assert lib.polar_hip_fadd(None, None, 1.0, None, 1.0, None, 4) == 1
+    assert lib.polar_hip_fmatmul(None, 0, 0, None, None, None, 1, 1, 1) == 1
+    assert b"dev is null" in lib.polar_hip_last_error()
+
+
+def _c(h):
+    c = h.counters()
+    return {n: getattr(c, n) for n, _ in c._fields_}
+
+
+def test_virtual_addresses_start_at_one_and_pack_by_bytes():
+    # src/core/context/internal/ContextInternal.cpp:24,43-48; e.g. 1, 17, 33 for 2x2 f32
+    with harness.Harness(plugin=None) as h:
+        assert [h.tensor(2, 2).vaddr for _ in range(3)] == [1, 17, 33]
+
+
+def test_call_sequence_and_coherence_on_mock():
+    with harness.Harness(plugin=None) as h:
+        assert h.device_name == "mock"
+        a = h.input(np.arange(8, dtype=np.float32))
+        b = h.input(np.ones(8, dtype=np.float32))
+        h.end_cluster()
+        c = h.fadd(a, 1.0, b, 1.0)
+        d = h.fmul(c, a)        # c is already on the device: no copy; a already uploaded
+        h.end_cluster()
+        h.run()
+        k = _c(h)
+        assert k["launches"] == 2
+        assert k["copies_to_device"] == 2 and k["bytes_to_device"] == 64  # a and b once each
+        assert k["copies_to_host"] == 0                                  # nothing read yet
+        assert k["events_waited"] == 2
+        # per node: releases of the READ args and of the result ride on the event
+        assert k["deferred_releases"] == 3 + 3
+        h.read(d)
+        h.read(d)                # the second read finds RAM up to date? no: RW bumped the version
+        k = _c(h)
+        assert k["copies_to_host"] == 1
+        # inputs were never written on the device: reading them needs no copy
+        assert np.array_equal(h.read(a), np.arange(8, dtype=np.float32))
+        assert _c(h)["copies_to_host"] == 1
+
+
+def test_host_write_invalidates_device_copy():
+    with harness.Harness(plugin=None) as h:
+        t = h.tensor(4)
+        h.host_write(t, [1, 2, 3, 4])
+        h.lock(t, 0, harness.READ); h.release(t, 0)
+        assert _c(h)["copies_to_device"] == 1
+        h.lock(t, 0, harness.READ); h.release(t, 0)
+        assert _c(h)["copies_to_device"] == 1      # still current
+        h.host_write(t, [5, 6, 7, 8])
+        h.lock(t, 0, harness.READ); h.release(t, 0)
+        assert _c(h)["copies_to_device"] == 2      # stale after the host write
+        h.lock(t, 0, harness.READ_WRITE); h.release(t, 0)
+        assert np.array_equal(h.read(t), [5, 6, 7, 8])  # mock copies real bytes
+        assert _c(h)["copies_to_host"] == 1
+
+
+def test_many_read_locks_are_allowed():
+    with harness.Harness(plugin=None) as h:
+        t = h.tensor(4)
+        h.host_write(t, [1, 2, 3, 4])
+        h.lock(t, 0, harness.READ)
+        h.lock(t, 0, harness.READ)
+        h.lock(t, harness.HOST, harness.READ)
+        h.release(t, 0); h.release(t, 0); h.release(t, harness.HOST)
+        h.lock(t, 0, harness.READ_WRITE)  # all released: allowed again
+        h.release(t, 0)
+
+
+def test_double_allocate_is_a_noop():
+    with harness.Harness(plugin=None) as h:
+        t = h.tensor(4)
+        h.allocate(t, 0); h.allocate(t, 0); h.allocate(t, harness.HOST)
+
+
+def test_usage_errors_return_minus_one():
+    with harness.Harness(plugin=None) as h:
+        t = h.tensor(4)
+        with pytest.raises(ValueError):
+            h.node("fadd", [t, 1.0, t, 1.0, 2.0], 4)   # result must be a tensor
+        with pytest.raises(ValueError):
+            h.node("fadd", [harness.Tensor(999, (4,)), 1.0, t, 1.0, t], 4)  # unknown tensor
+
+
+def _dies(code):
+    env = dict(os.environ, PYTHONPATH=REPO_ROOT)
+    prog = ("import __graft_entry__ as e; e.load_package();"
+            "from polarai_framework_amd import harness; import numpy as np;"
+            "h = harness.Harness(plugin=None);" + code)
+    return subprocess.run([sys.executable, "-c", prog], env=env, capture_output=True, text=True, timeout=60)
+
+
+def test_read_write_lock_on_locked_tensor_is_fatal():
+    # tests/unit/backend/generic/lib/allocators/LayerAllocator.cpp:99-102 (ASSERT_DEATH)
+    r = _dies("t = h.tensor(4); h.host_write(t, [1,2,3,4]); h.lock(t, 0, 0); h.lock(t, 0, 1)")
+    assert r.returncode == 4  # ATH_BAD_ACCESS
+    assert "Attempt get READ_WRITE lock for tensor that is already locked" in r.stderr
+
+
+def test_host_read_write_lock_on_locked_tensor_is_fatal():
+    r = _dies("t = h.tensor(4); h.host_write(t, [1,2,3,4]); h.lock(t, 0, 0); h.lock(t, -1, 1)")
+    assert r.returncode == 4
+    assert "already locked" in r.stderr
+
+
+def test_plugin_without_devices_is_reported():
+    if capi.device_count() != 0:
+        pytest.skip("a GPU is present")
+    with pytest.raises(RuntimeError):
+        harness.Harness(plugin=LIB_PLUGIN)
