@@ -1,14 +1,20 @@
 // Memory-bound builtin operations for gfx950: fadd fmul fdivide fsigmoid
 // flogloss fmulconcat fcopy ffill.
 //
-// One kernel template serves all of them.  A work-group of 256 lanes owns a
-// tile of 256*UNROLL 16-byte vectors; every lane issues all of its dwordx4
-// loads before the first use so that UNROLL*NIN loads per lane are in flight,
-// then computes and stores.  Loads and stores are marked non-temporal: every
-// byte is touched once, so keeping it in L2 / Infinity Cache only evicts other
-// data.  Tiles are handed out grid-stride so any element count fits the grid.
-// The n % 4 trailing elements are done by the first lanes of block 0.  Buffers
-// that are not 16-byte aligned take a dword kernel instead.
+// One kernel template serves all of them.  A work-group of BLOCK lanes owns a
+// tile of BLOCK*UNROLL 16-byte vectors; every lane issues all of its dwordx4
+// loads before the first use, then computes and stores.  Measured on MI355X
+// with buffers rotated to defeat the Infinity Cache, the best shape for a
+// streaming kernel is the smallest one: one vector per lane (UNROLL = 1) and
+// work-groups of two waves for kernels that read (one wave-pair per 2 KiB of
+// each stream), four waves for the store-only fill (fewer, larger groups keep
+// the dispatcher ahead of the stores); grid-stride loops with a fixed grid
+// were 3-10 % slower.  Loads and stores are marked non-temporal: every byte
+// is touched once, so keeping it in L2 / Infinity Cache only evicts other
+// data (6-10 % faster than plain accesses).  Tiles are handed out grid-stride
+// only when the element count exceeds what one grid can index.  The n % 4
+// trailing elements are done by the first lanes of block 0.  Buffers that are
+// not 16-byte aligned take a dword kernel instead.
 //
 // Arithmetic is written so that it rounds exactly like the host kernels it
 // replaces: this file is compiled with -ffp-contract=off (no fused
@@ -22,7 +28,7 @@ namespace {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kBlock = 256;
+constexpr int kScalarBlock = 256;
 
 // ---- per-element operations ---------------------------------------------------
 // NIN = number of input streams.  apply(x, y) receives the i-th element of each.
@@ -106,7 +112,7 @@ template <> struct OpLoader<ScaleOp> {
   }
 };
 
-template <typename Op, int UNROLL>
+template <typename Op, int kBlock, int UNROLL>
 __global__ __launch_bounds__(kBlock) void ewVecKernel(
     Op op0, const float* scalarSrc, const v4f* a, const v4f* b, v4f* c,
     uint64_t n4, uint64_t n, uint64_t numTiles) {
@@ -158,12 +164,12 @@ __global__ __launch_bounds__(kBlock) void ewVecKernel(
 
 // Buffers with only 4-byte alignment: one dword per lane per step.
 template <typename Op>
-__global__ __launch_bounds__(kBlock) void ewScalarKernel(
+__global__ __launch_bounds__(kScalarBlock) void ewScalarKernel(
     Op op0, const float* scalarSrc, const float* a, const float* b, float* c,
     uint64_t n) {
   const Op op = OpLoader<Op>::load(op0, scalarSrc);
-  const uint64_t stride = uint64_t(gridDim.x) * kBlock;
-  for (uint64_t i = uint64_t(blockIdx.x) * kBlock + threadIdx.x; i < n;
+  const uint64_t stride = uint64_t(gridDim.x) * kScalarBlock;
+  for (uint64_t i = uint64_t(blockIdx.x) * kScalarBlock + threadIdx.x; i < n;
        i += stride) {
     float x = Op::NIN >= 1 ? a[i] : 0.0f;
     float y = Op::NIN >= 2 ? b[i] : 0.0f;
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(kBlock) void ewScalarKernel(
   }
 }
 
-template <typename Op, int UNROLL>
+template <typename Op, int kBlock = 128, int UNROLL = 1>
 int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
              const float* a, const float* b, float* c, uint64_t n) {
   if (n == 0) return POLAR_HIP_OK;
@@ -183,17 +189,17 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
     constexpr uint64_t kTile = uint64_t(kBlock) * UNROLL;
     const uint64_t numTiles = (n4 + kTile - 1) / kTile;
     uint64_t grid = numTiles < 1 ? 1 : numTiles;
-    if (grid > (1u << 22)) grid = 1u << 22;
-    ewVecKernel<Op, UNROLL><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
+    if (grid > (1u << 30)) grid = 1u << 30;
+    ewVecKernel<Op, kBlock, UNROLL><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
                               dev->stream>>>(
         op, scalarSrc, reinterpret_cast<const v4f*>(a),
         reinterpret_cast<const v4f*>(b), reinterpret_cast<v4f*>(c), n4, n,
         numTiles);
   } else {
-    uint64_t grid = (n + kBlock - 1) / kBlock;
+    uint64_t grid = (n + kScalarBlock - 1) / kScalarBlock;
     const uint64_t cap = uint64_t(dev->info.compute_units) * 32;
     if (grid > cap) grid = cap;
-    ewScalarKernel<Op><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
+    ewScalarKernel<Op><<<dim3(static_cast<unsigned>(grid)), dim3(kScalarBlock), 0,
                          dev->stream>>>(op, scalarSrc, a, b, c, n);
   }
   POLAR_HIP_TRY(hipGetLastError());
@@ -208,21 +214,21 @@ int polar_hip_fadd(polar_hip_device* dev, const float* a, float scaleA,
                    const float* b, float scaleB, float* c, uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (a && b && c), "null tensor");
-  return launchEw<AddOp, 4>(dev, AddOp{scaleA, scaleB}, nullptr, a, b, c, n);
+  return launchEw<AddOp>(dev, AddOp{scaleA, scaleB}, nullptr, a, b, c, n);
 }
 
 int polar_hip_fmul(polar_hip_device* dev, const float* a, const float* b,
                    float* c, uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (a && b && c), "null tensor");
-  return launchEw<MulOp, 4>(dev, MulOp{}, nullptr, a, b, c, n);
+  return launchEw<MulOp>(dev, MulOp{}, nullptr, a, b, c, n);
 }
 
 int polar_hip_fdivide(polar_hip_device* dev, const float* numerator,
                       const float* denominator, float* out, uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (numerator && denominator && out), "null tensor");
-  return launchEw<DivOp, 4>(dev, DivOp{}, nullptr, numerator, denominator, out,
+  return launchEw<DivOp>(dev, DivOp{}, nullptr, numerator, denominator, out,
                             n);
 }
 
@@ -230,14 +236,14 @@ int polar_hip_fsigmoid(polar_hip_device* dev, const float* in, float* out,
                        uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (in && out), "null tensor");
-  return launchEw<SigmoidOp, 4>(dev, SigmoidOp{}, nullptr, in, nullptr, out, n);
+  return launchEw<SigmoidOp>(dev, SigmoidOp{}, nullptr, in, nullptr, out, n);
 }
 
 int polar_hip_flogloss(polar_hip_device* dev, const float* predicted,
                        const float* groundTruth, float* out, uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (predicted && groundTruth && out), "null tensor");
-  return launchEw<LogLossOp, 4>(dev, LogLossOp{}, nullptr, predicted,
+  return launchEw<LogLossOp>(dev, LogLossOp{}, nullptr, predicted,
                                 groundTruth, out, n);
 }
 
@@ -246,7 +252,7 @@ int polar_hip_fmulconcat(polar_hip_device* dev, const float* gradient,
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (gradient && localDerivative && out),
                     "null tensor");
-  return launchEw<ScaleOp, 4>(dev, ScaleOp{0.0f}, gradient, localDerivative,
+  return launchEw<ScaleOp>(dev, ScaleOp{0.0f}, gradient, localDerivative,
                               nullptr, out, n);
 }
 
@@ -254,14 +260,14 @@ int polar_hip_fcopy(polar_hip_device* dev, const float* src, float* dst,
                     uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || (src && dst), "null tensor");
-  return launchEw<CopyOp, 4>(dev, CopyOp{}, nullptr, src, nullptr, dst, n);
+  return launchEw<CopyOp>(dev, CopyOp{}, nullptr, src, nullptr, dst, n);
 }
 
 int polar_hip_ffill(polar_hip_device* dev, float pattern, float* out,
                     uint64_t n) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_REQUIRE(n == 0 || out, "null tensor");
-  return launchEw<FillOp, 4>(dev, FillOp{pattern}, nullptr, nullptr, nullptr,
+  return launchEw<FillOp, 256, 1>(dev, FillOp{pattern}, nullptr, nullptr, nullptr,
                              out, n);
 }
 
