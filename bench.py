@@ -9,8 +9,11 @@ steps.  After the timed region the same run measures ftranspose 12345x6789,
 the 4096^3 fp32 matmul in all four transpose variants, and the CPU oracle on
 the host cores (a reported baseline only).
 
-Per-kernel durations come from HIP events recorded on the library's own
-stream around every launch inside the timed region.
+Per-kernel durations come from HIP events attached to every launch inside the
+timed region on the library's own stream (each pair takes the kernel's own
+begin and end timestamps), so they are comparable with a profiler's kernel
+durations; `value` and `ms_per_step` use the host wall clock around the region
+and therefore include launch gaps.
 
 Prints ONE JSON line on stdout; progress goes to stderr.
 """
@@ -96,10 +99,8 @@ def main():
     def step(events=None):
         for op in SWEEP:
             if events is not None:
-                events.append(dev.record())
+                events.append(dev.time_next_kernel())
             launch(op)
-        if events is not None:
-            events.append(dev.record())
 
     for _ in range(args.warmup):
         step()
@@ -116,10 +117,9 @@ def main():
 
     per_op_ms = {op: [] for op in SWEEP}
     for ev in all_events:
-        for i, op in enumerate(SWEEP):
-            per_op_ms[op].append(ev[i].elapsed_ms(ev[i + 1]))
-        for e in ev:
-            e.release()
+        for (e0, e1), op in zip(ev, SWEEP):
+            per_op_ms[op].append(e0.elapsed_ms(e1))
+            e0.release(); e1.release()
     step_bytes = sum(BYTES_PER_ELEMENT[op] * n for op in SWEEP)
     value = step_bytes * args.steps / wall / 1e9
 
@@ -177,9 +177,8 @@ def time_kernel(dev, fn, warmup, reps):
     dev.synchronize()
     ms = []
     for _ in range(reps):
-        e0 = dev.record()
+        e0, e1 = dev.time_next_kernel()
         fn()
-        e1 = dev.record()
         e1.synchronize()
         ms.append(e0.elapsed_ms(e1))
         e0.release(); e1.release()

@@ -112,6 +112,13 @@ int polar_hip_stream_wait_event(polar_hip_device* dev, polar_hip_event* evt);
 /* Milliseconds between two completed events recorded on the same device. */
 int polar_hip_event_elapsed_ms(polar_hip_event* start, polar_hip_event* stop,
                                float* ms);
+/* Profiling aid with no counterpart in the reference: the next kernel that an
+ * entry point below launches on `dev` carries *start and *stop as its own
+ * begin and end timestamps, so polar_hip_event_elapsed_ms(*start, *stop) is
+ * that kernel's execution time without launch or queue gaps.  Synchronize
+ * *stop before reading; release both events afterwards. */
+int polar_hip_time_next_kernel(polar_hip_device* dev, polar_hip_event** start,
+                               polar_hip_event** stop);
 int polar_hip_event_release(polar_hip_event* evt);
 
 /* ---- builtin-operation kernels ---------------------------------------------

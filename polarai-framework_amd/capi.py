@@ -71,6 +71,7 @@ SIGNATURES = {
     "polar_hip_event_query": (_i, [_vp, C.POINTER(_i)]),
     "polar_hip_stream_wait_event": (_i, [_vp, _vp]),
     "polar_hip_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),
+    "polar_hip_time_next_kernel": (_i, [_vp, C.POINTER(_vp), C.POINTER(_vp)]),
     "polar_hip_event_release": (_i, [_vp]),
     "polar_hip_fadd": (_i, [_vp, _vp, _f, _vp, _f, _vp, _u64]),
     "polar_hip_fmul": (_i, [_vp, _vp, _vp, _vp, _u64]),
@@ -236,6 +237,12 @@ class Device:
         h = _vp()
         _check(self.lib, self.lib.polar_hip_event_record(self.handle, C.byref(h)))
         return Event(self, h)
+
+    def time_next_kernel(self):
+        """(start, stop) events that take the next kernel's own begin and end."""
+        s, e = _vp(), _vp()
+        _check(self.lib, self.lib.polar_hip_time_next_kernel(self.handle, C.byref(s), C.byref(e)))
+        return Event(self, s), Event(self, e)
 
     def wait_event(self, evt):
         _check(self.lib, self.lib.polar_hip_stream_wait_event(self.handle, evt.handle))

@@ -190,19 +190,19 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
     const uint64_t numTiles = (n4 + kTile - 1) / kTile;
     uint64_t grid = numTiles < 1 ? 1 : numTiles;
     if (grid > (1u << 30)) grid = 1u << 30;
-    ewVecKernel<Op, kBlock, UNROLL><<<dim3(static_cast<unsigned>(grid)), dim3(kBlock), 0,
-                              dev->stream>>>(
-        op, scalarSrc, reinterpret_cast<const v4f*>(a),
-        reinterpret_cast<const v4f*>(b), reinterpret_cast<v4f*>(c), n4, n,
-        numTiles);
+    POLAR_HIP_TRY(launchKernel(dev, ewVecKernel<Op, kBlock, UNROLL>,
+                               dim3(static_cast<unsigned>(grid)), dim3(kBlock), op,
+                               scalarSrc, reinterpret_cast<const v4f*>(a),
+                               reinterpret_cast<const v4f*>(b),
+                               reinterpret_cast<v4f*>(c), n4, n, numTiles));
   } else {
     uint64_t grid = (n + kScalarBlock - 1) / kScalarBlock;
     const uint64_t cap = uint64_t(dev->info.compute_units) * 32;
     if (grid > cap) grid = cap;
-    ewScalarKernel<Op><<<dim3(static_cast<unsigned>(grid)), dim3(kScalarBlock), 0,
-                         dev->stream>>>(op, scalarSrc, a, b, c, n);
+    POLAR_HIP_TRY(launchKernel(dev, ewScalarKernel<Op>,
+                               dim3(static_cast<unsigned>(grid)),
+                               dim3(kScalarBlock), op, scalarSrc, a, b, c, n));
   }
-  POLAR_HIP_TRY(hipGetLastError());
   return POLAR_HIP_OK;
 }
 

@@ -4,6 +4,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -32,6 +33,11 @@ struct polar_hip_device {
   std::vector<polar_hip_event*> idleEvents;
   std::vector<polar_hip_event*> allEvents;
 
+  // armed by polar_hip_time_next_kernel: the next kernel launch carries these
+  // as its start/stop events
+  polar_hip_event* timeStart = nullptr;
+  polar_hip_event* timeStop = nullptr;
+
 };
 
 namespace polar_hip_detail {
@@ -39,6 +45,25 @@ namespace polar_hip_detail {
 int fail(polar_hip_status st, const char* fmt, ...)
     __attribute__((format(printf, 2, 3)));
 int failHip(hipError_t e, const char* what);
+
+// Every kernel of the library is launched through here.  Normally a plain
+// launch on the device's stream; when a timing pair is armed, the launch
+// carries the pair so that the events take the kernel's own begin and end
+// timestamps (no host or queue gaps in between).
+template <typename... KArgs, typename... Args>
+inline hipError_t launchKernel(polar_hip_device* dev, void (*kernel)(KArgs...),
+                               dim3 grid, dim3 block, Args... args) {
+  if (dev->timeStart != nullptr) {
+    hipEvent_t e0 = dev->timeStart->ev, e1 = dev->timeStop->ev;
+    dev->timeStart = dev->timeStop = nullptr;
+    hipExtLaunchKernelGGL(kernel, grid, block, 0, dev->stream, e0, e1, 0,
+                          static_cast<KArgs>(args)...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, 0, dev->stream,
+                       static_cast<KArgs>(args)...);
+  }
+  return hipGetLastError();
+}
 
 inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;

@@ -255,15 +255,14 @@ int launchLayout(polar_hip_device* dev, const MatmulArgs& p0, bool vec,
     return fail(POLAR_HIP_ERR_INVALID, "fmatmul: too many tiles");
   const dim3 grid(static_cast<unsigned>(groups)), block(WM * WN * 64);
   if (vec && !edge)
-    matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, false>
-        <<<grid, block, 0, dev->stream>>>(p);
+    POLAR_HIP_TRY(launchKernel(
+        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, false>, grid, block, p));
   else if (vec && edge)
-    matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, true>
-        <<<grid, block, 0, dev->stream>>>(p);
+    POLAR_HIP_TRY(launchKernel(
+        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, true>, grid, block, p));
   else
-    matmulKernel<BM, BN, BK, WM, WN, TA, TB, false, true>
-        <<<grid, block, 0, dev->stream>>>(p);
-  POLAR_HIP_TRY(hipGetLastError());
+    POLAR_HIP_TRY(launchKernel(
+        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, false, true>, grid, block, p));
   return POLAR_HIP_OK;
 }
 

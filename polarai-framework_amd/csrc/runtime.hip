@@ -298,6 +298,34 @@ int polar_hip_event_elapsed_ms(polar_hip_event* start, polar_hip_event* stop,
   return POLAR_HIP_OK;
 }
 
+// Arms a start/stop pair for the next kernel launched on `dev`.
+int polar_hip_time_next_kernel(polar_hip_device* dev, polar_hip_event** start,
+                               polar_hip_event** stop) {
+  POLAR_HIP_REQUIRE(dev && start && stop, "null argument");
+  *start = *stop = nullptr;
+  polar_hip_event* pair[2] = {nullptr, nullptr};
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  for (auto*& e : pair) {
+    {
+      std::lock_guard<std::mutex> g(dev->mu);
+      if (!dev->idleEvents.empty()) {
+        e = dev->idleEvents.back();
+        dev->idleEvents.pop_back();
+      }
+    }
+    if (e == nullptr) {
+      hipEvent_t he;
+      POLAR_HIP_TRY(hipEventCreate(&he));
+      e = new polar_hip_event{dev, he};
+      std::lock_guard<std::mutex> g(dev->mu);
+      dev->allEvents.push_back(e);
+    }
+  }
+  dev->timeStart = *start = pair[0];
+  dev->timeStop = *stop = pair[1];
+  return POLAR_HIP_OK;
+}
+
 int polar_hip_event_release(polar_hip_event* evt) {
   POLAR_HIP_REQUIRE(evt != nullptr, "evt is null");
   std::lock_guard<std::mutex> g(evt->dev->mu);

@@ -83,9 +83,9 @@ extern "C" int polar_hip_ftranspose(polar_hip_device* dev, const float* in,
   uint64_t grid = numTiles;
   if (grid > (1u << 22)) grid = 1u << 22;
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-  transposeKernel<<<dim3(static_cast<unsigned>(grid)), dim3(kThreads), 0,
-                    dev->stream>>>(in, out, rows, cols,
-                                   static_cast<uint32_t>(tilesX), numTiles);
-  POLAR_HIP_TRY(hipGetLastError());
+  POLAR_HIP_TRY(launchKernel(dev, transposeKernel,
+                             dim3(static_cast<unsigned>(grid)), dim3(kThreads),
+                             in, out, rows, cols, static_cast<uint32_t>(tilesX),
+                             numTiles));
   return POLAR_HIP_OK;
 }

@@ -226,12 +226,3 @@ def test_mismatched_matmul_shapes_are_fatal():
     r = _dies("a = h.input(np.ones((4, 5), dtype=np.float32)); b = h.input(np.ones((6, 3), dtype=np.float32));"
               "h.end_cluster(); h.node('fmatmul_f_f', [a, b, h.tensor(4, 3)], 2); h.end_cluster(); h.run()")
     assert r.returncode != 0 and "shapes do not agree" in r.stderr
-
-
-def test_non_fp32_tensor_is_fatal_in_support_routines():
-    # src/backend/generic/runtime/support/routines.cpp:94-96: double is refused
-    # (the mini-executor only declares fp32 tensors, so this is reached through
-    # the device library's own argument checks instead)
-    r = _dies("t = h.tensor(4); h.node('ffill', [1.0, t], 1); h.end_cluster(); h.run();"
-              "print(h.read(t))")
-    assert r.returncode == 0 and "1. 1. 1. 1." in r.stdout

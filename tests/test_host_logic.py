@@ -91,7 +91,7 @@ def test_call_sequence_and_coherence_on_mock():
         # per node: releases of the READ args and of the result ride on the event
         assert k["deferred_releases"] == 3 + 3
         h.read(d)
-        h.read(d)                # the second read finds RAM up to date? no: RW bumped the version
+        h.read(d)                # RAM now holds the newest version: no second copy
         k = _c(h)
         assert k["copies_to_host"] == 1
         # inputs were never written on the device: reading them needs no copy
