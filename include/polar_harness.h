@@ -93,6 +93,14 @@ int polar_harness_release(polar_harness* h, uint64_t vaddr, int device);
 int polar_harness_host_write(polar_harness* h, uint64_t vaddr, const float* data,
                              uint64_t count);
 
+/* Raw object pointers (Device* of the device under test, the BackendAllocator*,
+ * the plugin's Context* or NULL for the mock), for code that wants to use them
+ * through its own declaration of the interface -- the interface-conformance
+ * probe built from the framework's headers does. */
+void* polar_harness_raw_device(polar_harness* h);
+void* polar_harness_raw_allocator(polar_harness* h);
+void* polar_harness_raw_context(polar_harness* h);
+
 int polar_harness_get_counters(polar_harness* h, polar_harness_counters* out);
 /* Cap the device layer's capacity (bytes; 0 = no cap) to force the offload
  * path.  Returns -1 if the selected device is not the HIP plugin's. */

@@ -1,0 +1,140 @@
+// Caller-side probe of the runtime-plugin interface, compiled against the
+// REFERENCE's own headers (-I<reference>/include), never against this
+// repository's restatement of them.  TEST INFRASTRUCTURE ONLY.
+//
+// Each function takes objects that were created by code built with
+// include/polar_rt_abi.hpp (the plugin's devices, the mini-executor's mock
+// device and allocator) and uses them through the reference's class
+// declarations.  If the restated vtable order, a by-value parameter type or a
+// struct layout differed from the reference's, these calls would land in the
+// wrong function or read the wrong field, and the tests that drive this probe
+// would fail.
+//
+// Only headers that compile straight from the reference tree are used
+// (Context/Device/Event/AllocatorLayerBase/MemoryRecord/ProgramDesc,
+// LaunchCommand.h, TensorInfo.h).  BackendAllocator.hpp is not: it needs the
+// cmake-generated polar_core_export.h, so a BackendAllocator only passes
+// through here as an opaque reference.
+#include <cstddef>
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include <polarai/backend/generic/runtime/Context.hpp>
+#include <polarai/backend/generic/runtime/Event.hpp>
+#include <polarai/backend/generic/runtime/LaunchCommand.h>
+#include <polarai/backend/generic/runtime/TensorInfo.h>
+
+using namespace polarai::backend::generic;
+
+extern "C" {
+
+// sizeof / offsetof of the plain structs as the reference declares them
+void ref_struct_layout(uint64_t* out /* 12 values */) {
+  out[0] = sizeof(TensorInfo);
+  out[1] = offsetof(TensorInfo, virtAddr);
+  out[2] = offsetof(TensorInfo, dataType);
+  out[3] = offsetof(TensorInfo, dims);
+  out[4] = offsetof(TensorInfo, shape);
+  out[5] = sizeof(ArgDesc);
+  out[6] = offsetof(ArgDesc, arg);
+  out[7] = offsetof(ArgDesc, type);
+  out[8] = sizeof(LaunchCommand);
+  out[9] = offsetof(LaunchCommand, argsCount);
+  out[10] = offsetof(LaunchCommand, nativeKernelName);
+  out[11] = sizeof(MemoryRecord);
+}
+
+int ref_context_device_count(void* context) {
+  return static_cast<int>(static_cast<Context*>(context)->getDevices().size());
+}
+
+void* ref_context_device(void* context, int index) {
+  return static_cast<Context*>(context)->getDevices().at(index).get();
+}
+
+// Device information through the reference's vtable.
+// out: provider, kind, hasAllocator, isPartitionSupported(EQUALLY),
+//      partition(EQUALLY).size(), (device == device), (device != device)
+void ref_device_info(void* device, char* name, size_t nameLen, int* out) {
+  auto* d = static_cast<Device*>(device);
+  const std::string n = d->getDeviceName();
+  std::strncpy(name, n.c_str(), nameLen - 1);
+  name[nameLen - 1] = 0;
+  out[0] = static_cast<int>(d->getProvider());
+  out[1] = static_cast<int>(d->getKind());
+  out[2] = d->hasAllocator();
+  out[3] = d->isPartitionSupported(Device::PartitionDomain::EQUALLY);
+  out[4] = static_cast<int>(d->partition(Device::PartitionDomain::EQUALLY).size());
+  out[5] = (*d == *d);
+  out[6] = (*d != *d);
+  out[7] = static_cast<int>(std::hash<Device>()(*d) == std::hash<std::string>()(n));
+  std::vector<std::shared_ptr<ProgramDesc>> none;
+  d->selectBinary(none); // must be callable and do nothing harmful
+}
+
+// Allocator layer round trip through the reference's vtable, and a host ->
+// device -> host copy through Device::copyToDevice / copyToHost.
+// Returns 0 if every step behaved, otherwise the number of the failing step.
+int ref_allocator_and_copy(void* device, size_t vaddr, const float* src, float* dst,
+                           size_t count) {
+  auto* d = static_cast<Device*>(device);
+  std::shared_ptr<AllocatorLayerBase> layer = d->getAllocator();
+  if (!layer) return 1;
+  MemoryRecord rec{vaddr, count * sizeof(float)};
+  if (layer->isAllocated(rec)) return 2;
+  layer->allocate(rec);
+  if (!layer->isAllocated(rec)) return 3;
+  if (layer->getTag(rec) != 1) return 4;           // allocate sets tag 1
+  layer->allocate(rec);                              // double allocation: no-op
+  layer->setTag(rec, 7);
+  if (layer->getTag(rec) != 7) return 5;
+  if (layer->getPtr(rec) == nullptr) return 6;
+  layer->lock(rec);
+  d->copyToDevice(rec, const_cast<float*>(src));
+  d->copyToHost(rec, dst);
+  layer->release(rec);
+  layer->deallocate(rec);
+  if (layer->isAllocated(rec)) return 7;
+  int called = 0;
+  layer->registerMemoryOffloadCallback([&called](MemoryRecord, AllocatorLayerBase&) { ++called; });
+  return 0;
+}
+
+// Launch through Device::launch with structs laid out by the reference's
+// headers, then Event::addCallback / wait / getDevice and consumeEvent.
+// `allocator` is a BackendAllocator built elsewhere (opaque here).  Tensors
+// must already be allocated and locked on the device by the caller.
+// Returns 0 on success, else the failing step.
+int ref_launch_fadd(void* device, void* allocator, uint64_t va, uint64_t vb, uint64_t vc,
+                    uint64_t count, float scaleA, float scaleB) {
+  auto* d = static_cast<Device*>(device);
+  uint64_t shape[1] = {count};
+  TensorInfo ta{va, 2, 1, shape}, tb{vb, 2, 1, shape}, tc{vc, 2, 1, shape};
+  ArgDesc args[5];
+  args[0] = ArgDesc{0, &ta, ArgDesc::TENSOR};
+  args[1] = ArgDesc{sizeof(float), &scaleA, ArgDesc::DATA};
+  args[2] = ArgDesc{0, &tb, ArgDesc::TENSOR};
+  args[3] = ArgDesc{sizeof(float), &scaleB, ArgDesc::DATA};
+  args[4] = ArgDesc{0, &tc, ArgDesc::TENSOR};
+  LaunchCommand cmd{"probe_fadd", 5, args, "fadd"};
+  Event* evt = d->launch(*static_cast<BackendAllocator*>(allocator), cmd, nullptr);
+  if (evt == nullptr) return 1;
+  int ran = 0;
+  evt->addCallback([&ran]() { ++ran; });
+  if (ran != 0) return 2;            // callbacks run in wait(), not before
+  evt->wait();
+  if (ran != 1) return 3;
+  evt->wait();                       // callbacks run once
+  if (ran != 1) return 4;
+  if (evt->getDevice() == nullptr) return 5;
+  // a second launch that depends on the first event
+  Event* evt2 = d->launch(*static_cast<BackendAllocator*>(allocator), cmd, evt);
+  if (evt2 == nullptr) return 6;
+  d->consumeEvent(evt2);             // waits and gives the event back
+  return 0;
+}
+
+} // extern "C"

@@ -46,6 +46,9 @@ SIGNATURES = {
     "polar_harness_lock": (_i, [_vp, _u64, _i, _i]),
     "polar_harness_release": (_i, [_vp, _u64, _i]),
     "polar_harness_host_write": (_i, [_vp, _u64, _vp, _u64]),
+    "polar_harness_raw_device": (_vp, [_vp]),
+    "polar_harness_raw_allocator": (_vp, [_vp]),
+    "polar_harness_raw_context": (_vp, [_vp]),
     "polar_harness_get_counters": (_i, [_vp, C.POINTER(Counters)]),
     "polar_harness_set_device_byte_limit": (_i, [_vp, _u64]),
 }
@@ -232,6 +235,15 @@ class Harness:
     def host_write(self, t, data):
         data = np.ascontiguousarray(data, dtype=np.float32)
         self._ok(self.lib.polar_harness_host_write(self.h, t.vaddr, data.ctypes.data, data.size), "host_write")
+
+    def raw_device(self):
+        return self.lib.polar_harness_raw_device(self.h)
+
+    def raw_allocator(self):
+        return self.lib.polar_harness_raw_allocator(self.h)
+
+    def raw_context(self):
+        return self.lib.polar_harness_raw_context(self.h)
 
     def counters(self):
         c = Counters()

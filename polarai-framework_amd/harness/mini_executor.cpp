@@ -335,6 +335,12 @@ int polar_harness_host_write(polar_harness* h, uint64_t vaddr, const float* data
   return 0;
 }
 
+void* polar_harness_raw_device(polar_harness* h) { return h ? h->inner.get() : nullptr; }
+void* polar_harness_raw_allocator(polar_harness* h) {
+  return h ? static_cast<BackendAllocator*>(h->allocator.get()) : nullptr;
+}
+void* polar_harness_raw_context(polar_harness* h) { return h ? h->ctx : nullptr; }
+
 int polar_harness_get_counters(polar_harness* h, polar_harness_counters* out) {
   if (h == nullptr || out == nullptr) return -1;
   *out = h->counters;

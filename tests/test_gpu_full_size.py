@@ -1,0 +1,106 @@
+"""Parity at the benchmark's full sizes: the elementwise sweep at 2^26
+elements against the oracle (all host threads), the 4096^3 matmul in all four
+transpose variants against sampled oracle rows plus size-independent
+identities, and the ragged elementwise / transpose shapes."""
+import numpy as np
+import pytest
+
+import parity
+import polar_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+N = 1 << 26
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _all_threads():
+    o.set_threads(o.hw_threads())
+    yield
+    o.set_threads(1)
+
+
+def test_elementwise_sweep_full_size(dev):
+    rng = np.random.default_rng(20240607)
+    a = parity.uniform(rng, N, -1, 1)
+    b = parity.uniform(rng, N, -1, 1)
+    den = parity.uniform(rng, N, 0.5, 2)
+    da, db, dden, dout = dev.array(a), dev.array(b), dev.array(den), dev.empty(N)
+    print("fadd", flush=True)
+    dev.fadd(da, 1.0, db, 1.0, dout)
+    assert np.array_equal(dout.download(), o.fadd(a, 1.0, b, 1.0))
+    dev.fadd(da, 0.34, db, 0.21, dout)
+    assert np.array_equal(dout.download(), o.fadd(a, 0.34, b, 0.21))
+    print("fmul", flush=True)
+    dev.fmul(da, db, dout)
+    assert np.array_equal(dout.download(), o.fmul(a, b))
+    print("fdivide", flush=True)
+    dev.fdivide(da, dden, dout)
+    assert np.array_equal(dout.download(), o.fdivide(a, den))
+    print("fcopy / ffill", flush=True)
+    dev.fcopy(da, dout)
+    assert np.array_equal(dout.download(), a)
+    dev.ffill(3.0, dout)
+    got = dout.download()
+    assert got.min() == 3.0 and got.max() == 3.0
+    print("fsigmoid / flogloss", flush=True)
+    dev.fsigmoid(da, dout)
+    p = dout.download()
+    assert parity.elementwise_rel_error(p, o.fsigmoid(a)) <= parity.ELEMENTWISE_REL
+    y = (b > 0.8).astype(np.float32)  # Bernoulli(0.1) labels
+    db.upload(y)
+    dev.flogloss(dout, db, dden)
+    assert parity.elementwise_rel_error(dden.download(), o.flogloss(p, y)) <= parity.ELEMENTWISE_REL
+    for x in (da, db, dden, dout):
+        x.free()
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_4096_cubed(dev, ta, tb):
+    m = n = k = 4096
+    rng = np.random.default_rng(6 + 2 * ta + tb)
+    a = parity.normal(rng, (k, m) if ta else (m, k))
+    b = parity.normal(rng, (n, k) if tb else (k, n))
+    da, db, dc = dev.array(a), dev.array(b), dev.empty(m * n)
+    dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+    got = dc.download((m, n))
+    # oracle on 3 bands of 8 rows: first, middle (tile boundary), last
+    for r0 in (0, 2044, 4088):
+        print("oracle rows", r0, flush=True)
+        ref = o.fmatmul(ta, tb, a, b, rows=(r0, r0 + 8))[r0:r0 + 8]
+        assert parity.frobenius_rel_error(got[r0:r0 + 8], ref) <= parity.MATMUL_FRO_REL
+    # whole result: linearity probe  C x = A (B x)  in fp64 for a random x
+    x = rng.standard_normal(n)
+    A = (a.T if ta else a).astype(np.float64)
+    B = (b.T if tb else b).astype(np.float64)
+    lhs, rhs = got.astype(np.float64) @ x, A @ (B @ x)
+    assert np.linalg.norm(lhs - rhs) / np.linalg.norm(rhs) < 1e-5
+    # and against the transposed problem (B^T A^T = C^T), computed on the device
+    dct = dev.empty(m * n)
+    dev.fmatmul(not tb, not ta, db, da, dct, n, m, k)
+    assert parity.frobenius_rel_error(dct.download((n, m)).T, got) <= parity.MATMUL_FRO_REL
+    for t in (da, db, dc, dct):
+        t.free()
+
+
+def test_ragged_elementwise_and_transpose(dev):
+    n = 1000003
+    rng = np.random.default_rng(77)
+    a, b = parity.uniform(rng, n, -1, 1), parity.uniform(rng, n, -1, 1)
+    for mis in (0, 1):
+        da, db, dc = dev.array(a, mis), dev.array(b, mis), dev.empty(n, mis)
+        dev.fadd(da, 1.0, db, 1.0, dc)
+        assert np.array_equal(dc.download(), o.fadd(a, 1.0, b, 1.0))
+        dev.fmul(da, db, dc)
+        assert np.array_equal(dc.download(), o.fmul(a, b))
+        for t in (da, db, dc):
+            t.free()
+    x = parity.normal(rng, (12345, 6789))
+    dx, dt, dtt = dev.array(x), dev.empty(x.size), dev.empty(x.size)
+    dev.ftranspose(dx, dt, 12345, 6789)
+    assert np.array_equal(dt.download((6789, 12345)), o.ftranspose(x))
+    dev.ftranspose(dt, dtt, 6789, 12345)
+    assert np.array_equal(dtt.download((12345, 6789)), x)
+    for t in (dx, dt, dtt):
+        t.free()
