@@ -24,6 +24,12 @@
 // Shapes that are not multiples of the tile, leading dimensions that are not
 // multiples of 4 and unaligned base pointers are handled by predicated /
 // scalar fetch variants chosen on the host.
+//
+// Shapes whose C has too few tiles to occupy the chip (skinny outputs, long
+// K) are split along K: every split writes its partial product to a workspace
+// from the device pool and a second kernel adds the partials in split order,
+// so the result does not depend on scheduling.  Tile shape and split count
+// come from a small cost model (planMatmul) of rounds x k-steps x step time.
 #include "internal.h"
 
 using namespace polar_hip_detail;
@@ -39,9 +45,11 @@ constexpr int kXcds = 8;
 struct MatmulArgs {
   const float* A;
   const float* B;
-  float* C;
+  float* C;        // final output, or the workspace when kSplits > 1
   uint32_t M, N, K;
   uint32_t tilesM, tilesN;
+  uint32_t kSplits;   // work-groups [s*tiles, (s+1)*tiles) handle split s
+  uint32_t kPerSplit; // multiple of BK
 };
 
 // Fetch of one operand tile (BX x BK) from HBM into registers, and its store
@@ -166,9 +174,14 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
   const int wave = t / 64;
   const int wm = wave / WN, wn = wave % WN;
 
+  const uint32_t tiles = p.tilesM * p.tilesN;
+  const uint32_t split = blockIdx.x / tiles;
   uint32_t tm, tn;
-  tileOfGroup(blockIdx.x, gridDim.x, p.tilesM, p.tilesN, tm, tn);
+  tileOfGroup(blockIdx.x % tiles, tiles, p.tilesM, p.tilesN, tm, tn);
   const uint32_t m0 = tm * BM, n0 = tn * BN;
+  const uint32_t kBegin = split * p.kPerSplit;
+  const uint32_t kEnd = kBegin + p.kPerSplit < p.K ? kBegin + p.kPerSplit : p.K;
+  float* const out = p.C + size_t(split) * p.M * p.N;
 
   // A: k-contiguous when not transposed ([M x K]); B: k-contiguous when
   // transposed ([N x K]).
@@ -185,9 +198,9 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  const uint32_t nk = (p.K + BK - 1) / BK;
-  fa.load(p.A, lda, m0, 0, p.M, p.K, t);
-  fb.load(p.B, ldb, n0, 0, p.N, p.K, t);
+  const uint32_t nk = kEnd > kBegin ? (kEnd - kBegin + BK - 1) / BK : 0;
+  fa.load(p.A, lda, m0, kBegin, p.M, kEnd, t);
+  fb.load(p.B, ldb, n0, kBegin, p.N, kEnd, t);
   fa.store(As[0], t);
   fb.store(Bs[0], t);
   __syncthreads();
@@ -200,8 +213,8 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
     const int cur = kt & 1;
     const bool more = kt + 1 < nk;
     if (more) {
-      fa.load(p.A, lda, m0, (kt + 1) * BK, p.M, p.K, t);
-      fb.load(p.B, ldb, n0, (kt + 1) * BK, p.N, p.K, t);
+      fa.load(p.A, lda, m0, kBegin + (kt + 1) * BK, p.M, kEnd, t);
+      fb.load(p.B, ldb, n0, kBegin + (kt + 1) * BK, p.N, kEnd, t);
     }
     const float* as = As[cur];
     const float* bs = Bs[cur];
@@ -238,19 +251,27 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
         const uint32_t row =
             m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
         if (!EDGE || (row < p.M && col < p.N))
-          p.C[size_t(row) * p.N + col] = acc[i][j][r];
+          out[size_t(row) * p.N + col] = acc[i][j][r];
       }
     }
   }
 }
 
+// C[i] = partial[0][i] + partial[1][i] + ... in split order.
+__global__ __launch_bounds__(256) void splitKReduceKernel(const float* __restrict__ partial,
+                                                          float* __restrict__ c,
+                                                          uint64_t count, uint32_t splits) {
+  const uint64_t stride = uint64_t(gridDim.x) * 256;
+  for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) {
+    float acc = partial[i];
+    for (uint32_t s = 1; s < splits; ++s) acc += partial[uint64_t(s) * count + i];
+    c[i] = acc;
+  }
+}
+
 template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
-int launchLayout(polar_hip_device* dev, const MatmulArgs& p0, bool vec,
-                 bool edge) {
-  MatmulArgs p = p0;
-  p.tilesM = (p.M + BM - 1) / BM;
-  p.tilesN = (p.N + BN - 1) / BN;
-  const uint64_t groups = uint64_t(p.tilesM) * p.tilesN;
+int launchLayout(polar_hip_device* dev, const MatmulArgs& p, bool vec, bool edge) {
+  const uint64_t groups = uint64_t(p.tilesM) * p.tilesN * p.kSplits;
   if (groups >= (1ull << 31))
     return fail(POLAR_HIP_ERR_INVALID, "fmatmul: too many tiles");
   const dim3 grid(static_cast<unsigned>(groups)), block(WM * WN * 64);
@@ -267,7 +288,14 @@ int launchLayout(polar_hip_device* dev, const MatmulArgs& p0, bool vec,
 }
 
 template <int BM, int BN, int BK, int WM, int WN>
-int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p) {
+int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
+               uint32_t splits) {
+  MatmulArgs p = p0;
+  p.tilesM = (p.M + BM - 1) / BM;
+  p.tilesN = (p.N + BN - 1) / BN;
+  const uint32_t kSteps = (p.K + BK - 1) / BK;
+  p.kSplits = splits;
+  p.kPerSplit = (kSteps + splits - 1) / splits * BK;
   // 16-byte fetches need aligned bases and a contiguous dimension that is a
   // multiple of 4 for both operands.
   const uint32_t contigA = ta ? p.M : p.K;
@@ -275,10 +303,88 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p) {
   const bool vec = aligned16(p.A) && aligned16(p.B) && contigA % 4 == 0 &&
                    contigB % 4 == 0;
   const bool edge = p.M % BM != 0 || p.N % BN != 0 || p.K % BK != 0;
-  if (!ta && !tb) return launchLayout<BM, BN, BK, WM, WN, false, false>(dev, p, vec, edge);
-  if (!ta && tb) return launchLayout<BM, BN, BK, WM, WN, false, true>(dev, p, vec, edge);
-  if (ta && !tb) return launchLayout<BM, BN, BK, WM, WN, true, false>(dev, p, vec, edge);
-  return launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
+
+  float* const c = p.C;
+  void* workspace = nullptr;
+  const uint64_t count = uint64_t(p.M) * p.N;
+  if (splits > 1) {
+    int st = polar_hip_alloc(dev, count * splits * sizeof(float), &workspace);
+    if (st != POLAR_HIP_OK) return st;
+    p.C = static_cast<float*>(workspace);
+  }
+  int st;
+  if (!ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, false, false>(dev, p, vec, edge);
+  else if (!ta && tb) st = launchLayout<BM, BN, BK, WM, WN, false, true>(dev, p, vec, edge);
+  else if (ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, true, false>(dev, p, vec, edge);
+  else st = launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
+  if (splits > 1) {
+    if (st == POLAR_HIP_OK) {
+      uint64_t grid = (count + 255) / 256;
+      const uint64_t cap = uint64_t(dev->info.compute_units) * 16;
+      if (grid > cap) grid = cap;
+      hipError_t e = launchKernel(dev, splitKReduceKernel, dim3(static_cast<unsigned>(grid)),
+                                  dim3(256), static_cast<const float*>(workspace), c, count,
+                                  splits);
+      if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
+    }
+    // stream-ordered pool: the block may be handed out again only to work
+    // enqueued after the reduction
+    polar_hip_free(dev, workspace);
+  }
+  return st;
+}
+
+// ---- tile shape and split count -----------------------------------------------
+struct TileConfig {
+  int bm, bn, bk, waves, residentGroups;
+  float mfmaEfficiency; // fraction of the matrix pipe a lone group can use
+};
+// order = the switch in polar_hip_fmatmul
+constexpr TileConfig kConfigs[] = {
+    {128, 128, 16, 4, 2, 0.85f}, // 2x2 waves of 64x64
+    {64, 64, 16, 4, 4, 0.60f},   // 2x2 waves of 32x32
+    {128, 32, 32, 4, 2, 0.55f},  // skinny N
+    {32, 128, 32, 4, 2, 0.55f},  // skinny M
+    {32, 32, 32, 1, 8, 0.15f},   // one wave
+};
+
+struct MatmulPlan {
+  int config;
+  uint32_t splits;
+};
+
+// Estimated microseconds = rounds x k-steps x step time (+ reduction).  A step
+// of a lone group is bound by the latency of its global->LDS->MFMA chain
+// (about 1.3 us, measured); co-resident groups overlap until they saturate the
+// CU's matrix pipe (256 flop/clk at 2.4 GHz).
+MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
+  static const uint32_t kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256};
+  MatmulPlan best{0, 1};
+  double bestUs = 1e30;
+  for (int c = 0; c < int(sizeof(kConfigs) / sizeof(kConfigs[0])); ++c) {
+    const TileConfig& t = kConfigs[c];
+    const double tiles = double((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
+    const uint32_t kSteps = (k + t.bk - 1) / t.bk;
+    const double mfmaUs = 2.0 * t.bm * t.bn * t.bk / (256.0 * 2400.0 * t.mfmaEfficiency);
+    for (uint32_t s : kSplitChoices) {
+      if (s > 1 && (kSteps / s < 2 || double(m) * n * s * 4 > double(256u << 20))) break;
+      const double groups = tiles * s;
+      double resident = groups / computeUnits;
+      if (resident < 1) resident = 1;
+      if (resident > t.residentGroups) resident = t.residentGroups;
+      const double rounds = groups <= double(computeUnits) * resident
+                                ? 1.0
+                                : groups / (double(computeUnits) * resident);
+      const double stepUs = resident * mfmaUs > 1.3 ? resident * mfmaUs : 1.3;
+      double us = rounds * ((kSteps + s - 1) / s) * stepUs + 3.0;
+      if (s > 1) us += 4.0 + double(m) * n * 4.0 * (s + 1) / 3.0e6;
+      if (us < bestUs) {
+        bestUs = us;
+        best = MatmulPlan{c, s};
+      }
+    }
+  }
+  return best;
 }
 
 } // namespace
@@ -299,10 +405,14 @@ extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
     return polar_hip_ffill(dev, 0.0f, c, m * n);
   }
   MatmulArgs p{a, b, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
-               static_cast<uint32_t>(k), 0, 0};
+               static_cast<uint32_t>(k), 0, 0, 1, 0};
   const bool ta = transA != 0, tb = transB != 0;
-  if (n <= 32) return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p);
-  if (m <= 32) return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p);
-  if (m <= 64 || n <= 64) return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p);
-  return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p);
+  const MatmulPlan plan = planMatmul(p.M, p.N, p.K, dev->info.compute_units);
+  switch (plan.config) {
+  case 0: return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 1: return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 2: return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p, plan.splits);
+  case 3: return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p, plan.splits);
+  default: return launchTile<32, 32, 32, 1, 1>(dev, ta, tb, p, plan.splits);
+  }
 }
