@@ -51,18 +51,25 @@ int failHip(hipError_t e, const char* what);
 // carries the pair so that the events take the kernel's own begin and end
 // timestamps (no host or queue gaps in between).
 template <typename... KArgs, typename... Args>
-inline hipError_t launchKernel(polar_hip_device* dev, void (*kernel)(KArgs...),
-                               dim3 grid, dim3 block, Args... args) {
+inline hipError_t launchKernelLds(polar_hip_device* dev, void (*kernel)(KArgs...),
+                                  dim3 grid, dim3 block, uint32_t dynamicLdsBytes,
+                                  Args... args) {
   if (dev->timeStart != nullptr) {
     hipEvent_t e0 = dev->timeStart->ev, e1 = dev->timeStop->ev;
     dev->timeStart = dev->timeStop = nullptr;
-    hipExtLaunchKernelGGL(kernel, grid, block, 0, dev->stream, e0, e1, 0,
-                          static_cast<KArgs>(args)...);
+    hipExtLaunchKernelGGL(kernel, grid, block, dynamicLdsBytes, dev->stream, e0, e1,
+                          0, static_cast<KArgs>(args)...);
   } else {
-    hipLaunchKernelGGL(kernel, grid, block, 0, dev->stream,
+    hipLaunchKernelGGL(kernel, grid, block, dynamicLdsBytes, dev->stream,
                        static_cast<KArgs>(args)...);
   }
   return hipGetLastError();
+}
+
+template <typename... KArgs, typename... Args>
+inline hipError_t launchKernel(polar_hip_device* dev, void (*kernel)(KArgs...),
+                               dim3 grid, dim3 block, Args... args) {
+  return launchKernelLds(dev, kernel, grid, block, 0u, args...);
 }
 
 inline bool aligned16(const void* p) {

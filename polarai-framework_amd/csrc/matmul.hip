@@ -17,6 +17,16 @@
 // LDS words per lane and issues TM*TN MFMAs.  LDS row pitch is BX + 4 words so
 // the scattered stores of the k-contiguous case spread over the banks.
 //
+// What bounds the 4096^3 case on MI355X (measured): the matrix pipes need 2^31
+// busy cycles over 1024 SIMDs; under this kernel's LDS and L2 traffic the chip
+// clocks at 2.0-2.2 GHz instead of 2.4, and a SIMD that interleaves MFMAs of
+// four waves sustains only 80 % of the rate it reaches with one or two (124 vs
+// 155 TFLOP/s in a register-only loop).  A hand-pipelined variant (three LDS
+// stages, register prefetch two steps ahead, fragments read one k-pair ahead,
+// occupancy capped at two waves per SIMD) landed on the same plateau and was
+// dropped; larger tiles (less LDS and L2 traffic per flop) gained 5-7 %, hence
+// the 256 x 256 x 32 configuration for big shapes.
+//
 // Work-groups are numbered so that the groups resident on one XCD (which share
 // an L2) cover a compact block of C tiles and therefore re-use the same rows
 // of A and columns of B.
@@ -31,6 +41,7 @@
 // so the result does not depend on scheduling.  Tile shape and split count
 // come from a small cost model (planMatmul) of rounds x k-steps x step time.
 #include "internal.h"
+
 
 using namespace polar_hip_detail;
 
@@ -272,8 +283,6 @@ __global__ __launch_bounds__(256) void splitKReduceKernel(const float* __restric
 template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
 int launchLayout(polar_hip_device* dev, const MatmulArgs& p, bool vec, bool edge) {
   const uint64_t groups = uint64_t(p.tilesM) * p.tilesN * p.kSplits;
-  if (groups >= (1ull << 31))
-    return fail(POLAR_HIP_ERR_INVALID, "fmatmul: too many tiles");
   const dim3 grid(static_cast<unsigned>(groups)), block(WM * WN * 64);
   if (vec && !edge)
     POLAR_HIP_TRY(launchKernel(
@@ -341,7 +350,8 @@ struct TileConfig {
 };
 // order = the switch in polar_hip_fmatmul
 constexpr TileConfig kConfigs[] = {
-    {128, 128, 16, 4, 2, 0.85f}, // 2x2 waves of 64x64
+    {256, 256, 32, 16, 1, 0.92f}, // 4x4 waves of 64x64: one group per CU
+    {128, 128, 16, 4, 2, 0.85f},  // 2x2 waves of 64x64
     {64, 64, 16, 4, 4, 0.60f},   // 2x2 waves of 32x32
     {128, 32, 32, 4, 2, 0.55f},  // skinny N
     {32, 128, 32, 4, 2, 0.55f},  // skinny M
@@ -359,7 +369,7 @@ struct MatmulPlan {
 // CU's matrix pipe (256 flop/clk at 2.4 GHz).
 MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
   static const uint32_t kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256};
-  MatmulPlan best{0, 1};
+  MatmulPlan best{1, 1};
   double bestUs = 1e30;
   for (int c = 0; c < int(sizeof(kConfigs) / sizeof(kConfigs[0])); ++c) {
     const TileConfig& t = kConfigs[c];
@@ -409,10 +419,11 @@ extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
   const bool ta = transA != 0, tb = transB != 0;
   const MatmulPlan plan = planMatmul(p.M, p.N, p.K, dev->info.compute_units);
   switch (plan.config) {
-  case 0: return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 1: return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 2: return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p, plan.splits);
-  case 3: return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p, plan.splits);
+  case 0: return launchTile<256, 256, 32, 4, 4>(dev, ta, tb, p, plan.splits);
+  case 1: return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 2: return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 3: return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p, plan.splits);
+  case 4: return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p, plan.splits);
   default: return launchTile<32, 32, 32, 1, 1>(dev, ta, tb, p, plan.splits);
   }
 }
