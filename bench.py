@@ -37,6 +37,15 @@ BYTES_PER_ELEMENT = {"fadd": 12, "fmul": 12, "fdivide": 12, "fsigmoid": 8,
                      "fcopy": 8, "ffill": 4, "flogloss": 12, "fmulconcat": 8,
                      "ftranspose": 8}
 SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
+# HBM-side bytes per launch at the sizes below, from two `rocprofv3 --pmc` runs
+# of this script (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by
+# what the same counter reads for the plain copy kernel fcopy
+# (profiles/bench_kernels_pmc_traffic.md).  They cannot be measured from inside
+# this process, so they are constants of the committed kernels.
+MEASURED_TRAFFIC_BYTES = {
+    "fadd": 805166953, "fmul": 805157993, "fdivide": 805155989, "fsigmoid": 536769637,
+    "fcopy": 536870912, "ffill": 268482969, "ftranspose": 776973224, "fmatmul": 469770774,
+}
 T_ROWS, T_COLS = 12345, 6789
 MM = 4096
 
@@ -62,6 +71,8 @@ def main():
                     help="elements per tensor in the sweep (default 2^26)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-matmul", action="store_true", help="skip the matmul/transpose legs")
+    ap.add_argument("--no-graphs", action="store_true",
+                    help="skip the model-graph legs (keeps a profile to one problem size per kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this runtime drives one GPU; --gpus must be 1 "
@@ -128,12 +139,15 @@ def main():
         ms = float(np.mean(per_op_ms[op]))
         gbs = BYTES_PER_ELEMENT[op] * n / (ms * 1e-3) / 1e9
         per_op[op] = {"ms": round(ms, 5), "min_ms": round(float(np.min(per_op_ms[op])), 5),
-                      "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+                      "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                      "algorithmic_bytes": BYTES_PER_ELEMENT[op] * n,
+                      "traffic": MEASURED_TRAFFIC_BYTES[op] if n == N_SWEEP else None}
         log(f"{op:10s} {ms * 1e3:9.1f} us  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of HBM peak")
     dominant = max(SWEEP, key=lambda op: np.mean(per_op_ms[op]))
     roofline = {"bound": "hbm", "kernel": dominant,
                 "achieved": per_op[dominant]["GB/s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(per_op[dominant]["GB/s"] / HBM_PEAK_GBS, 4), "traffic": None}
+                "frac": round(per_op[dominant]["GB/s"] / HBM_PEAK_GBS, 4),
+                "traffic": per_op[dominant]["traffic"]}
 
     # quick sanity of what was timed (full parity lives in tests/)
     probe = outs["fadd"].download()[:1024]
@@ -163,11 +177,16 @@ def main():
         result["transpose"] = bench_transpose(dev, args)
         result["matmul"] = bench_matmul(dev, args)
     da.free(); db.free()
+    dev.close()
+    dev = None
+    if not args.no_graphs:
+        result["graphs"] = bench_graphs()
 
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, b, den, n)
 
-    dev.close()
+    if dev is not None:
+        dev.close()
     print(json.dumps(result), flush=True)
 
 
@@ -199,7 +218,8 @@ def bench_transpose(dev, args):
     return {"workload": f"ftranspose {T_ROWS}x{T_COLS} fp32", "ms": round(float(np.mean(ms)), 5),
             "min_ms": round(float(np.min(ms)), 5), "GB/s": round(gbs, 1),
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
-                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}}
+                         "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
+                         "traffic": MEASURED_TRAFFIC_BYTES["ftranspose"]}}
 
 
 def bench_matmul(dev, args):
@@ -235,7 +255,63 @@ def bench_matmul(dev, args):
     out["GFLOP/s"] = round(mean_tf * 1e3, 1)
     out["roofline"] = {"bound": "mfma", "achieved": round(mean_tf, 2), "peak": MFMA_FP32_PEAK_TFLOPS,
                        "unit": "TFLOP/s", "frac": round(mean_tf / MFMA_FP32_PEAK_TFLOPS, 4),
-                       "worst_variant_frac": round(worst / MFMA_FP32_PEAK_TFLOPS, 4), "traffic": None}
+                       "worst_variant_frac": round(worst / MFMA_FP32_PEAK_TFLOPS, 4),
+                       "traffic": MEASURED_TRAFFIC_BYTES["fmatmul"]}
+    return out
+
+
+def bench_graphs():
+    """The two model configurations as kernel DAGs through the runtime plugin
+    (initContext -> Device::launch per node, barrier per cluster): latency-bound
+    at these sizes, so wall-clock per evaluation is what is reported."""
+    from polarai_framework_amd import LIB_PLUGIN, graphs, harness
+    out = {}
+    rng = np.random.default_rng(61)
+    x = rng.random((256, 784), dtype=np.float32)
+    w = (rng.standard_normal((784, 10)) * 0.01).astype(np.float32)
+    bias = np.zeros((256, 10), dtype=np.float32)
+    y = (rng.random((256, 10)) < 0.1).astype(np.float32)
+    g, _ = graphs.logreg_forward(x, w, bias, y)
+    with harness.Harness(plugin=LIB_PLUGIN) as h:
+        graphs.emit(g, h, {})
+        for _ in range(5):
+            h.run()
+        ts = []
+        for _ in range(50):
+            t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
+        c = h.counters()
+        out["logreg_forward"] = {
+            "workload": "X[256x784] W[784x10]: 4 input nodes, fmatmul_f_f -> fadd -> fsigmoid -> flogloss, "
+                        "one barrier per cluster, inputs re-loaded every evaluation as the framework does",
+            "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
+            "launches_per_evaluate": 4, "uploads_per_evaluate": int(c.copies_to_device // 55)}
+        log(f"logreg forward through the plugin: {out['logreg_forward']['evaluate_us']} us per evaluation")
+    rng = np.random.default_rng(71)
+    x = rng.random((1024, 1024), dtype=np.float32)
+    w1 = (rng.standard_normal((1024, 4096)) / 32).astype(np.float32)
+    w2 = (rng.standard_normal((4096, 1024)) / 64).astype(np.float32)
+    y = (rng.random((1024, 1024)) < 0.5).astype(np.float32)
+    f, gr, u, _ = graphs.mlp_graphs(x, w1, w2, y)
+    with harness.Harness(plugin=LIB_PLUGIN) as h:
+        tensors = {}
+        times = {}
+        for graph in (f, gr, u):
+            graphs.emit(graph, h, tensors)
+            h.run()  # first evaluation allocates
+            ts = []
+            for _ in range(3):
+                t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
+            times[graph.name] = float(np.median(ts))
+            h.clear_program()
+        out["mlp_forward_backward"] = {
+            "workload": "batch 1024, 1024->4096->1024, sigmoid, logloss; forward, the framework's gradient "
+                        "graph and its in-place weight update, each evaluated through the plugin",
+            "forward_ms": round(times["mlp_forward"] * 1e3, 3),
+            "gradient_ms": round(times["mlp_gradient"] * 1e3, 3),
+            "update_ms": round(times["mlp_update"] * 1e3, 3),
+            "nodes": {gph.name: len(gph.nodes) for gph in (f, gr, u)}}
+        log(f"mlp through the plugin: forward {times['mlp_forward'] * 1e3:.2f} ms, gradient "
+            f"{times['mlp_gradient'] * 1e3:.2f} ms, update {times['mlp_update'] * 1e3:.2f} ms")
     return out
 
 

@@ -2,6 +2,7 @@
 // library (the non-kernel half of include/polar_hip.h).
 #include "internal.h"
 
+#include <chrono>
 #include <cstdio>
 #include <cstring>
 
@@ -264,8 +265,19 @@ int polar_hip_event_record(polar_hip_device* dev, polar_hip_event** out) {
   return POLAR_HIP_OK;
 }
 
+// Graph code waits on an event after every cluster, typically for a kernel that
+// runs for microseconds, so the wake-up latency of a blocking wait is paid once
+// per node.  Poll for a short while first and only then block.
 int polar_hip_event_synchronize(polar_hip_event* evt) {
   POLAR_HIP_REQUIRE(evt != nullptr, "evt is null");
+  const auto t0 = std::chrono::steady_clock::now();
+  for (;;) {
+    hipError_t e = hipEventQuery(evt->ev);
+    if (e == hipSuccess) return POLAR_HIP_OK;
+    if (e != hipErrorNotReady) return failHip(e, "hipEventQuery");
+    (void)hipGetLastError();
+    if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(200)) break;
+  }
   POLAR_HIP_TRY(hipEventSynchronize(evt->ev));
   return POLAR_HIP_OK;
 }

@@ -207,6 +207,33 @@ def test_matmul_unaligned_base(dev, ta, tb):
     assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
 
 
+SPLIT_K_SHAPES = [(33, 127, 4099), (33, 127, 65536), (256, 10, 784), (10, 256, 2051), (64, 64, 8192),
+                  (130, 70, 3000), (1024, 1024, 4096)]
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("mnk", SPLIT_K_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_long_k_is_split_and_reduced_in_order(dev, ta, tb, mnk):
+    # few output tiles and a long K: the contraction is split along K and the
+    # partial products are added in split order
+    m, n, k = mnk
+    _say("split-k matmul", ta, tb, mnk)
+    o.set_threads(o.hw_threads())
+    try:
+        rng = np.random.default_rng(m + 3 * n + 5 * k + 2 * ta + tb)
+        sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+        a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+        got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+        rows = (0, m) if m * n * k < 3e8 else (m // 2 - 4, m // 2 + 4)
+        ref = o.fmatmul(ta, tb, a, b, rows=rows)
+        assert parity.frobenius_rel_error(got[rows[0]:rows[1]], ref[rows[0]:rows[1]]) <= parity.MATMUL_FRO_REL
+        again = _matmul_device(dev, ta, tb, a, b, m, n, k)
+        assert np.array_equal(got, again)  # deterministic: no atomics, fixed reduction order
+    finally:
+        o.set_threads(1)
+
+
 def test_matmul_overwrites_output(dev):
     # no beta: C is overwritten, stale contents must not leak
     rng = np.random.default_rng(31)
