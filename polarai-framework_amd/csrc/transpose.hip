@@ -7,53 +7,55 @@
 //  * Writes that cover only part of a 128-byte line are expensive (a plain
 //    64x64-tile kernel drops from 5.2 TB/s on a line-aligned shape to 2.5 TB/s
 //    on this one, and the write side accounts for most of it).  So the output
-//    is cut into 256-byte chunks that are aligned IN MEMORY, not in index
+//    is cut into 128-byte chunks that are aligned IN MEMORY, not in index
 //    space: for output row j the chunk boundaries sit at the i for which
-//    (j*rows + i) % 64 == 0, i.e. at b_j + 64m with b_j = (-j*rows) mod 64.
-//    Every wave-wide store then writes two whole lines; only the first and
-//    last chunk of an output row can be partial.
-//  * Because b_j differs from row to row, the 64 output rows of a work-group
-//    need input rows from a window that is up to 127 rows tall.  The group
-//    therefore walks down a strip of the input, 64 rows per step, keeping the
-//    last two 64x64 tiles in an LDS ring; step m emits, for every output row,
-//    the aligned chunk that ends inside tile m.  Each input element is read
-//    once per strip (plus one extra tile at the strip's end).
+//    (j*rows + i) % 32 == 0, i.e. at b_j + 32m with b_j = (-j*rows) mod 32.
+//    Every half-wave store then writes one whole line; only the first and last
+//    chunk of an output row can be partial.
+//  * Because b_j differs from row to row, the output rows of a work-group need
+//    input rows from a window that is up to 63 rows tall.  The group therefore
+//    walks down a strip of the input, 32 rows per step, keeping the last two
+//    32 x 256 tiles in an LDS ring; step m emits, for every output row, the
+//    aligned chunk that ends inside tile m.  Each input element is read once
+//    per strip (plus one extra tile at the strip's end).
 //  * Input row segments are not line-aligned either, so neighbouring column
-//    tiles share cache lines.  Work-groups are numbered so that each XCD owns a
-//    contiguous range of column tiles and walks them together: the shared
-//    lines then hit in that XCD's L2 instead of being fetched twice
-//    (3.7 -> 4.4 TB/s).
-//  * 1024 lanes per group (16 waves): 4 loads per lane in flight, and four
-//    output rows per wave in the store phase.
+//    tiles share cache lines.  Column tiles are 256 wide (1 KiB segments: two
+//    shared lines per nine) and work-groups are numbered so that each XCD owns
+//    a contiguous range of column tiles and walks them together: the shared
+//    lines then mostly hit in that XCD's L2 instead of being fetched twice.
+//  * 1024 lanes per group (16 waves): 8 loads per lane in flight, and 32 output
+//    rows per wave in the store phase, two per wave-wide store.
 //
-// The LDS ring has a row pitch of 65 words, so both the row-wise stores of the
-// load phase and the column-wise loads of the store phase are conflict-free.
-// All edges are predicated; any rows x cols works.
+// The LDS ring has a row pitch of 257 words, so both the row-wise stores of the
+// load phase and the column-wise loads of the store phase are conflict-free
+// within a half-wave.  All edges are predicated; any rows x cols works.
 #include "internal.h"
 
 using namespace polar_hip_detail;
 
 namespace {
 
-constexpr int kT = 64;          // tile edge: 64 input rows x 64 input columns
+constexpr int kTI = 32;   // input rows per step = elements per aligned output chunk
+constexpr int kTJ = 256;  // input columns (= output rows) per work-group
 constexpr int kThreads = 1024;
 constexpr int kWaves = kThreads / 64;
-constexpr int kRowsPerPass = kThreads / kT; // 16
-constexpr int kPasses = kT / kRowsPerPass;  // 4 loads per lane per tile
+constexpr int kLoads = kTI * kTJ / kThreads;    // 8 loads per lane per tile
+constexpr int kColsPerStore = 64 / kTI;         // 2 output rows per wave-wide store
+constexpr int kStores = kTJ / (kWaves * kColsPerStore); // 8 stores per lane per step
 constexpr int kXcds = 8;
 
 struct TransposeArgs {
   const float* in;
   float* out;
   uint32_t rows, cols;
-  uint32_t colTiles;        // ceil(cols / 64)
+  uint32_t colTiles;        // ceil(cols / kTJ)
   uint32_t colTilesPerXcd;  // ceil(colTiles / 8)
   uint32_t strips;          // ceil(rows / stripRows)
-  uint32_t stripRows;       // multiple of 64
+  uint32_t stripRows;       // multiple of kTI
 };
 
 __global__ __launch_bounds__(kThreads) void transposeKernel(TransposeArgs p) {
-  __shared__ float ring[2 * kT][kT + 1];
+  __shared__ float ring[2 * kTI][kTJ + 1];
 
   // XCD x (work-groups with id % 8 == x) owns column tiles
   // [x*perXcd, (x+1)*perXcd) and walks them fastest.
@@ -63,51 +65,56 @@ __global__ __launch_bounds__(kThreads) void transposeKernel(TransposeArgs p) {
   if (colTile >= p.colTiles || strip >= p.strips) return; // before any barrier
 
   const uint32_t R = p.rows, C = p.cols;
-  const uint32_t j0 = colTile * kT;
+  const uint32_t j0 = colTile * kTJ;
   const uint32_t i0 = strip * p.stripRows;
   const uint32_t i1 = i0 + p.stripRows < R ? i0 + p.stripRows : R;
   const bool lastStrip = i1 == R;
   // tiles 0..lastTile are loaded; the final one only feeds the chunks that
   // straddle the end of the strip
-  const uint32_t lastTile = lastStrip ? (R - i0 + kT - 1) / kT : (i1 - i0) / kT;
+  const uint32_t lastTile = lastStrip ? (R - i0 + kTI - 1) / kTI : (i1 - i0) / kTI;
 
   const int t = threadIdx.x;
-  const int tx = t % kT, ty = t / kT;
   const int wave = t / 64, lane = t % 64;
-  const bool colOk = j0 + tx < C;
+  const int sub = lane / kTI, l = lane % kTI;
 
-  float v[kPasses];
+  float v[kLoads];
   auto loadTile = [&](uint32_t m) {
 #pragma unroll
-    for (int q = 0; q < kPasses; ++q) {
-      const uint64_t r = uint64_t(i0) + uint64_t(m) * kT + ty + q * kRowsPerPass;
-      v[q] = (r < R && colOk) ? __builtin_nontemporal_load(&p.in[r * C + j0 + tx])
-                              : 0.0f;
+    for (int q = 0; q < kLoads; ++q) {
+      const int e = t + q * kThreads;
+      const int row = e / kTJ, col = e % kTJ;
+      const uint64_t r = uint64_t(i0) + uint64_t(m) * kTI + row;
+      v[q] = (r < R && j0 + col < C)
+                 ? __builtin_nontemporal_load(&p.in[r * C + j0 + col])
+                 : 0.0f;
     }
   };
 
   loadTile(0);
   for (uint32_t m = 0; m <= lastTile; ++m) {
-    const int half = (m & 1) * kT;
+    const int half = (m & 1) * kTI;
 #pragma unroll
-    for (int q = 0; q < kPasses; ++q) ring[half + ty + q * kRowsPerPass][tx] = v[q];
+    for (int q = 0; q < kLoads; ++q) {
+      const int e = t + q * kThreads;
+      ring[half + e / kTJ][e % kTJ] = v[q];
+    }
     __syncthreads();
     if (m < lastTile) loadTile(m + 1); // in flight during the store phase
 
     // Store phase: output row j0+c gets the aligned chunk that ends in tile m,
-    // i in [i0 + 64(m-1) + b, i0 + 64m + b), clipped to what this strip owns.
+    // i in [i0 + 32(m-1) + b, i0 + 32m + b), clipped to what this strip owns.
 #pragma unroll
-    for (int q = 0; q < kT / kWaves; ++q) {
-      const int c = wave + kWaves * q;
+    for (int q = 0; q < kStores; ++q) {
+      const int c = wave * kColsPerStore + sub + q * (kWaves * kColsPerStore);
       const uint32_t j = j0 + c;
       const uint64_t rowBase = uint64_t(j) * R;
-      const uint32_t b = uint32_t((64 - (rowBase & 63)) & 63);
-      const int64_t first = int64_t(i0) + int64_t(kT) * (int64_t(m) - 1) + b;
+      const uint32_t b = uint32_t((kTI - (rowBase & (kTI - 1))) & (kTI - 1));
+      const int64_t first = int64_t(i0) + int64_t(kTI) * (int64_t(m) - 1) + b;
       const int64_t own0 = i0 == 0 ? 0 : int64_t(i0) + b;
       const int64_t own1 = lastStrip ? int64_t(R) : int64_t(i1) + b;
-      const int64_t i = first + lane;
+      const int64_t i = first + l;
       if (j < C && i >= own0 && i < own1 && i < int64_t(R)) {
-        const float val = ring[uint32_t(i - i0) & (2 * kT - 1)][c];
+        const float val = ring[uint32_t(i - i0) & (2 * kTI - 1)][c];
         __builtin_nontemporal_store(val, &p.out[rowBase + uint64_t(i)]);
       }
     }
@@ -130,12 +137,12 @@ extern "C" int polar_hip_ftranspose(polar_hip_device* dev, const float* in,
   p.out = out;
   p.rows = static_cast<uint32_t>(rows);
   p.cols = static_cast<uint32_t>(cols);
-  p.colTiles = (p.cols + kT - 1) / kT;
+  p.colTiles = (p.cols + kTJ - 1) / kTJ;
   p.colTilesPerXcd = (p.colTiles + kXcds - 1) / kXcds;
   // Longest strip (fewest re-read tiles) that still gives every CU two groups.
   const uint64_t wanted = 2ull * static_cast<uint64_t>(dev->info.compute_units);
   uint32_t stripRows = 512;
-  while (stripRows > kT &&
+  while (stripRows > kTI &&
          uint64_t(p.colTiles) * ((p.rows + stripRows - 1) / stripRows) < wanted)
     stripRows /= 2;
   p.stripRows = stripRows;
