@@ -33,6 +33,10 @@ struct polar_hip_device {
   std::vector<polar_hip_event*> idleEvents;
   std::vector<polar_hip_event*> allEvents;
 
+  // pinned bounce buffer for small and medium host<->device copies
+  std::mutex stagingMu;
+  void* staging = nullptr;
+
   // armed by polar_hip_time_next_kernel: the next kernel launch carries these
   // as its start/stop events
   polar_hip_event* timeStart = nullptr;

@@ -109,6 +109,7 @@ int polar_hip_device_close(polar_hip_device* dev) {
     (void)hipEventDestroy(e->ev);
     delete e;
   }
+  if (dev->staging) (void)hipHostFree(dev->staging);
   (void)hipStreamDestroy(dev->stream);
   delete dev;
   return POLAR_HIP_OK;
@@ -207,6 +208,26 @@ int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out) {
 }
 
 // ---- copies -----------------------------------------------------------------
+// Host memory handed in by the framework is pageable.  The driver's pageable
+// path is fast for large transfers (30 GB/s up, 18 GB/s down, measured) but has
+// a high fixed cost for small and medium ones (110 us for 256 KiB), which is
+// what graph inputs and read-backs mostly are.  Those go through a pinned
+// bounce buffer instead: one host memcpy plus one DMA.
+namespace {
+constexpr uint64_t kStagingBytes = 4ull << 20;
+
+void* stagingBuffer(polar_hip_device* dev) {
+  if (dev->staging == nullptr) {
+    void* p = nullptr;
+    if (hipHostMalloc(&p, kStagingBytes, hipHostMallocDefault) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    dev->staging = p;
+  }
+  return dev->staging;
+}
+} // namespace
 
 int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
                              const void* src_host, uint64_t bytes) {
@@ -215,6 +236,16 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
   POLAR_HIP_REQUIRE(dst_device != nullptr && src_host != nullptr,
                     "null buffer");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  if (bytes <= kStagingBytes) {
+    std::lock_guard<std::mutex> g(dev->stagingMu);
+    if (void* pinned = stagingBuffer(dev)) {
+      memcpy(pinned, src_host, bytes);
+      POLAR_HIP_TRY(hipMemcpyAsync(dst_device, pinned, bytes, hipMemcpyHostToDevice,
+                                   dev->stream));
+      POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+      return POLAR_HIP_OK;
+    }
+  }
   POLAR_HIP_TRY(hipMemcpyAsync(dst_device, src_host, bytes,
                                hipMemcpyHostToDevice, dev->stream));
   POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
@@ -228,6 +259,16 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
   POLAR_HIP_REQUIRE(dst_host != nullptr && src_device != nullptr,
                     "null buffer");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  if (bytes <= kStagingBytes) {
+    std::lock_guard<std::mutex> g(dev->stagingMu);
+    if (void* pinned = stagingBuffer(dev)) {
+      POLAR_HIP_TRY(hipMemcpyAsync(pinned, src_device, bytes, hipMemcpyDeviceToHost,
+                                   dev->stream));
+      POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+      memcpy(dst_host, pinned, bytes);
+      return POLAR_HIP_OK;
+    }
+  }
   POLAR_HIP_TRY(hipMemcpyAsync(dst_host, src_device, bytes,
                                hipMemcpyDeviceToHost, dev->stream));
   POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
