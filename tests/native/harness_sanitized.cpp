@@ -1,0 +1,61 @@
+// Drives the mini-executor on its CPU mock device; built by
+// tests/test_native_sanitized.py together with the harness sources under
+// -fsanitize=address,undefined so that lifetime or indexing mistakes in the
+// host code show up without a GPU.
+#include "polar_harness.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#define CHECK(cond)                                                        \
+  do {                                                                     \
+    if (!(cond)) {                                                         \
+      std::fprintf(stderr, "%s:%d: check failed: %s\n", __FILE__, __LINE__, #cond); \
+      std::exit(1);                                                        \
+    }                                                                      \
+  } while (0)
+
+int main() {
+  for (int round = 0; round < 3; ++round) {
+    polar_harness* h = nullptr;
+    CHECK(polar_harness_open(nullptr, 0, &h) == 0);
+    CHECK(polar_harness_device_count(h) == 1);
+    const uint64_t shape[2] = {16, 8};
+    const uint64_t a = polar_harness_tensor(h, 2, shape);
+    const uint64_t b = polar_harness_tensor(h, 2, shape);
+    const uint64_t c = polar_harness_tensor(h, 2, shape);
+    const uint64_t d = polar_harness_tensor(h, 2, shape);
+    CHECK(a == 1 && b == 1 + 512 && c == 1 + 1024);
+    std::vector<float> data(128, 1.5f);
+    CHECK(polar_harness_input(h, a, data.data()) == 0);
+    CHECK(polar_harness_input(h, b, nullptr) == 0); // holder: loads nothing
+    CHECK(polar_harness_end_cluster(h) == 0);
+    polar_harness_arg add[5] = {{0, a, 0}, {1, 0, 1.0f}, {0, b, 0}, {1, 0, 2.0f}, {0, c, 0}};
+    CHECK(polar_harness_node(h, "fadd", 5, add, 4) == 0);
+    CHECK(polar_harness_end_cluster(h) == 0);
+    polar_harness_arg inplace[5] = {{0, c, 0}, {1, 0, 1.0f}, {0, a, 0}, {1, 0, 1.0f}, {0, a, 0}};
+    CHECK(polar_harness_node(h, "fadd", 5, inplace, 4) == 0); // result aliases an operand
+    polar_harness_arg mm[3] = {{0, a, 0}, {0, b, 0}, {0, d, 0}};
+    CHECK(polar_harness_node(h, "fmatmul_f_t", 3, mm, 2) == 0);
+    CHECK(polar_harness_node(h, "fadd", 5, add, 9) == -1);    // bad result index
+    CHECK(polar_harness_end_cluster(h) == 0);
+    for (int i = 0; i < 4; ++i) CHECK(polar_harness_run(h) == 0);
+    std::vector<float> out(128);
+    CHECK(polar_harness_read(h, c, out.data(), 128) == 0);
+    CHECK(polar_harness_read(h, a, out.data(), 129) == -1);   // too many elements
+    polar_harness_counters k;
+    CHECK(polar_harness_get_counters(h, &k) == 0);
+    CHECK(k.launches == 12 && k.events_waited == 12);
+    CHECK(polar_harness_clear_program(h) == 0);
+    CHECK(polar_harness_host_write(h, d, data.data(), 128) == 0);
+    CHECK(polar_harness_lock(h, d, 0, 0) == 0);
+    CHECK(polar_harness_release(h, d, 0) == 0);
+    CHECK(polar_harness_read(h, d, out.data(), 128) == 0);
+    CHECK(out[5] == 1.5f);
+    CHECK(polar_harness_raw_device(h) != nullptr && polar_harness_raw_context(h) == nullptr);
+    polar_harness_close(h);
+  }
+  std::puts("ok");
+  return 0;
+}
