@@ -13,8 +13,10 @@
 // is touched once, so keeping it in L2 / Infinity Cache only evicts other
 // data (6-10 % faster than plain accesses).  Tiles are handed out grid-stride
 // only when the element count exceeds what one grid can index.  The n % 4
-// trailing elements are done by the first lanes of block 0.  Buffers that are
-// not 16-byte aligned take a dword kernel instead.
+// trailing elements are done by the first lanes of block 0.  Streams that start
+// at the same offset from a 16-byte boundary are peeled by up to 31 leading
+// elements so that the output's vector stores cover whole 128-byte lines;
+// streams with different offsets take a dword kernel instead.
 //
 // Arithmetic is written so that it rounds exactly like the host kernels it
 // replaces: this file is compiled with -ffp-contract=off (no fused
@@ -112,11 +114,17 @@ template <> struct OpLoader<ScaleOp> {
   }
 };
 
+// as/bs/cs are the tensors themselves; the first `head` (< 32) elements bring
+// the output to a 128-byte line boundary (and every stream to a 16-byte one),
+// n4 vectors follow, then the tail.
 template <typename Op, int kBlock, int UNROLL>
 __global__ __launch_bounds__(kBlock) void ewVecKernel(
-    Op op0, const float* scalarSrc, const v4f* a, const v4f* b, v4f* c,
-    uint64_t n4, uint64_t n, uint64_t numTiles) {
+    Op op0, const float* scalarSrc, const float* as, const float* bs, float* cs,
+    uint32_t head, uint64_t n4, uint64_t n, uint64_t numTiles) {
   const Op op = OpLoader<Op>::load(op0, scalarSrc);
+  const v4f* a = reinterpret_cast<const v4f*>(as + head);
+  const v4f* b = reinterpret_cast<const v4f*>(bs + head);
+  v4f* c = reinterpret_cast<v4f*>(cs + head);
   constexpr uint64_t kTile = uint64_t(kBlock) * UNROLL;
   for (uint64_t tile = blockIdx.x; tile < numTiles; tile += gridDim.x) {
     const uint64_t base = tile * kTile + threadIdx.x;
@@ -149,15 +157,15 @@ __global__ __launch_bounds__(kBlock) void ewVecKernel(
       }
     }
   }
-  // trailing n % 4 elements
-  if (blockIdx.x == 0) {
-    const uint64_t i = n4 * 4 + threadIdx.x;
-    if (i < n) {
-      const float* as = reinterpret_cast<const float*>(a);
-      const float* bs = reinterpret_cast<const float*>(b);
+  // the elements before the first and after the last whole vector
+  if (blockIdx.x == 0 && threadIdx.x < 36) {
+    const uint64_t i = threadIdx.x < 32 ? threadIdx.x
+                                        : head + n4 * 4 + (threadIdx.x - 32);
+    const bool mine = threadIdx.x < 32 ? threadIdx.x < head : i < n;
+    if (mine) {
       float x = Op::NIN >= 1 ? as[i] : 0.0f;
       float y = Op::NIN >= 2 ? bs[i] : 0.0f;
-      reinterpret_cast<float*>(c)[i] = op.apply(x, y);
+      cs[i] = op.apply(x, y);
     }
   }
 }
@@ -182,19 +190,24 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
              const float* a, const float* b, float* c, uint64_t n) {
   if (n == 0) return POLAR_HIP_OK;
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-  const bool vec = aligned16(c) && (Op::NIN < 1 || aligned16(a)) &&
-                   (Op::NIN < 2 || aligned16(b));
+  // The vector path needs all streams to reach a 16-byte boundary after the
+  // same number of leading elements (always true for whole pool blocks).
+  const uintptr_t phase = reinterpret_cast<uintptr_t>(c) & 15u;
+  const bool vec = (Op::NIN < 1 || (reinterpret_cast<uintptr_t>(a) & 15u) == phase) &&
+                   (Op::NIN < 2 || (reinterpret_cast<uintptr_t>(b) & 15u) == phase);
   if (vec) {
-    const uint64_t n4 = n / 4;
+    // whole wave-wide stores should cover whole 128-byte lines of the output
+    uint32_t head = static_cast<uint32_t>(
+        ((128u - (reinterpret_cast<uintptr_t>(c) & 127u)) & 127u) / 4u);
+    if (head > n) head = static_cast<uint32_t>(n);
+    const uint64_t n4 = (n - head) / 4;
     constexpr uint64_t kTile = uint64_t(kBlock) * UNROLL;
     const uint64_t numTiles = (n4 + kTile - 1) / kTile;
     uint64_t grid = numTiles < 1 ? 1 : numTiles;
     if (grid > (1u << 30)) grid = 1u << 30;
     POLAR_HIP_TRY(launchKernel(dev, ewVecKernel<Op, kBlock, UNROLL>,
                                dim3(static_cast<unsigned>(grid)), dim3(kBlock), op,
-                               scalarSrc, reinterpret_cast<const v4f*>(a),
-                               reinterpret_cast<const v4f*>(b),
-                               reinterpret_cast<v4f*>(c), n4, n, numTiles));
+                               scalarSrc, a, b, c, head, n4, n, numTiles));
   } else {
     uint64_t grid = (n + kScalarBlock - 1) / kScalarBlock;
     const uint64_t cap = uint64_t(dev->info.compute_units) * 32;

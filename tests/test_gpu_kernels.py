@@ -24,7 +24,7 @@ def test_golden_vectors_on_device(dev, case):
 
 
 @pytest.mark.parametrize("n", SIZES)
-@pytest.mark.parametrize("misalign", [0, 1])
+@pytest.mark.parametrize("misalign", [0, 1, 3, 29])
 def test_binary_ops_bit_exact(dev, n, misalign):
     _say("binary ops n=", n, "misalign=", misalign)
     rng = np.random.default_rng(100 + n)
@@ -47,19 +47,24 @@ def test_binary_ops_bit_exact(dev, n, misalign):
 
 @pytest.mark.parametrize("n", SIZES)
 def test_mixed_alignment(dev, n):
-    # one operand 16-byte aligned, the other not: must take the dword path
+    # operands at different offsets from a 16-byte boundary: dword path;
+    # same offset modulo 16 bytes but different lines: vector path with a head
     _say("mixed alignment n=", n)
     rng = np.random.default_rng(200 + n)
     a, b = parity.uniform(rng, n, -1, 1), parity.uniform(rng, n, -1, 1)
-    da, db, dc = dev.array(a, 0), dev.array(b, 3), dev.empty(n, 2)
-    dev.fmul(da, db, dc)
-    assert np.array_equal(dc.download(), o.fmul(a, b))
-    for x in (da, db, dc):
-        x.free()
+    for ma, mb, mc in ((0, 3, 2), (1, 5, 9), (4, 0, 8), (7, 7, 7)):
+        da, db, dc = dev.array(a, ma), dev.array(b, mb), dev.empty(n + 8, mc)
+        dev.ffill(-7.0, dc, n + 8)
+        dev.fmul(da, db, dc, n)
+        got = dc.download()
+        assert np.array_equal(got[:n], o.fmul(a, b))
+        assert np.all(got[n:] == -7.0)          # nothing written past the end
+        for x in (da, db, dc):
+            x.free()
 
 
 @pytest.mark.parametrize("n", SIZES)
-@pytest.mark.parametrize("misalign", [0, 1])
+@pytest.mark.parametrize("misalign", [0, 1, 2, 31])
 def test_unary_and_fill(dev, n, misalign):
     _say("unary n=", n, "misalign=", misalign)
     rng = np.random.default_rng(300 + n)
