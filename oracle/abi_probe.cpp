@@ -19,15 +19,56 @@
 #include <cstdint>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include <polarai/backend/generic/runtime/Context.hpp>
 #include <polarai/backend/generic/runtime/Event.hpp>
+#include <polarai/backend/generic/runtime/GraphHandle.hpp>
 #include <polarai/backend/generic/runtime/LaunchCommand.h>
 #include <polarai/backend/generic/runtime/TensorInfo.h>
 
 using namespace polarai::backend::generic;
+
+// The support library under test (libpolar_rt_support_static.a, linked into
+// this probe).  The reference declares the seven routines in
+// src/backend/generic/runtime/support/api.hpp:18-32, which cannot be included
+// here (it needs a cmake-generated export header), so the prototypes are
+// written out with the reference's types; LockType is passed as the int the
+// lowering emits (READ = 0, READ_WRITE = 1 --
+// include/polarai/core/loader/internal/TensorAllocator.hpp:22).
+extern "C" {
+void ath_allocate(GraphHandle*, Device&, TensorInfo*);
+void ath_release(GraphHandle*, Device&, TensorInfo*, Event*);
+void ath_lock(GraphHandle*, Device&, TensorInfo*, int lockType);
+Device* ath_device_select(GraphHandle*, uint64_t nodeId);
+void ath_barrier(uint32_t count, Event** events);
+Event* ath_launch(GraphHandle*, Device*, Event*, LaunchCommand&);
+void ath_load(GraphHandle*, uint64_t nodeId, TensorInfo*);
+BackendAllocator* polar_rt_support_allocator_create();
+void polar_rt_support_allocator_destroy(BackendAllocator*);
+void polar_rt_support_register_device(BackendAllocator*, Device*);
+Device* polar_rt_support_host_device_create();
+void polar_rt_support_host_device_destroy(Device*);
+void polar_rt_support_graph_handle_layout(uint64_t out[5]);
+}
+
+namespace {
+// A loader as the support library documents it: a flat fp32 view of the
+// tensor.  `fill` copies data in; `drain` copies the tensor out (how this
+// probe reads results: the library hands the loader the RAM copy).
+struct FlatLoader {
+  virtual ~FlatLoader() = default;
+  virtual void load(float* dst, size_t count) {
+    if (fill != nullptr) std::memcpy(dst, fill, count * sizeof(float));
+    if (drain != nullptr) std::memcpy(drain, dst, count * sizeof(float));
+  }
+  const float* fill = nullptr;
+  float* drain = nullptr;
+};
+} // namespace
 
 extern "C" {
 
@@ -135,6 +176,105 @@ int ref_launch_fadd(void* device, void* allocator, uint64_t va, uint64_t vb, uin
   if (evt2 == nullptr) return 6;
   d->consumeEvent(evt2);             // waits and gives the event back
   return 0;
+}
+
+// sizeof(GraphHandle) and member offsets as the reference declares it, then
+// the same five numbers as the support library was compiled.
+void ref_graph_handle_layout(uint64_t* out) {
+  out[0] = sizeof(GraphHandle);
+  out[1] = offsetof(GraphHandle, allocator);
+  out[2] = offsetof(GraphHandle, devices);
+  out[3] = offsetof(GraphHandle, mLoaders);
+  out[4] = offsetof(GraphHandle, isHostNode);
+  polar_rt_support_graph_handle_layout(out + 5);
+}
+
+// One graph evaluation as JIT-compiled code performs it
+// (src/core/graph/internal/GraphCompiler.cpp:55-108), on a GraphHandle laid
+// out by the reference's header, through the support library's ath_*:
+// two input nodes (host), one fadd node on `device`, a barrier, then a host
+// read of the result (pulled from the device by the host lock) and of the
+// first input (whose RAM copy must have survived the device's READ lock).  `device` comes from a runtime plugin or is the mini-executor's mock
+// (which computes nothing: sum is then left untouched by the launch).
+// Returns 0 on success, else the failing step.
+int ref_support_evaluate(void* device, uint64_t count, const float* a, const float* b,
+                         float scaleA, float scaleB, float* sum, float* aBack) {
+  auto* dev = static_cast<Device*>(device);
+  BackendAllocator* rawAllocator = polar_rt_support_allocator_create();
+  Device* rawHost = polar_rt_support_host_device_create();
+  if (rawAllocator == nullptr || rawHost == nullptr) return 1;
+  polar_rt_support_register_device(rawAllocator, dev);
+
+  FlatLoader loadA, loadB, readSum, readA;
+  loadA.fill = a;
+  loadB.fill = b;
+  readSum.drain = sum;
+  readA.drain = aBack;
+  using Loader = polarai::core::internal::AbstractLoaderInternal;
+  int status = 0;
+  {
+    GraphHandle handle;
+    handle.allocator = std::shared_ptr<BackendAllocator>(
+        rawAllocator, [](BackendAllocator* p) { polar_rt_support_allocator_destroy(p); });
+    handle.devices.push_back(std::shared_ptr<Device>(dev, [](Device*) {})); // borrowed
+    handle.devices.push_back(
+        std::shared_ptr<Device>(rawHost, [](Device* p) { polar_rt_support_host_device_destroy(p); }));
+    handle.mLoaders[1] = reinterpret_cast<Loader*>(&loadA);
+    handle.mLoaders[2] = reinterpret_cast<Loader*>(&loadB);
+    handle.mLoaders[4] = reinterpret_cast<Loader*>(&readSum);
+    handle.mLoaders[5] = reinterpret_cast<Loader*>(&readA);
+    for (uint64_t id : {1, 2, 4, 5}) handle.isHostNode.insert(id);
+
+    uint64_t shape[1] = {count};
+    const uint64_t bytes = count * sizeof(float);
+    TensorInfo ta{1, 2, 1, shape}, tb{1 + bytes, 2, 1, shape}, tc{1 + 2 * bytes, 2, 1, shape};
+
+    // input nodes
+    for (auto [id, t] : {std::pair<uint64_t, TensorInfo*>{1, &ta}, {2, &tb}}) {
+      Device* host = ath_device_select(&handle, id);
+      if (host != rawHost) { status = 2; break; }
+      ath_allocate(&handle, *host, t);
+      ath_lock(&handle, *host, t, 1);
+      ath_load(&handle, id, t);
+      ath_release(&handle, *host, t, nullptr);
+    }
+    // fadd node
+    Event* evt = nullptr;
+    if (status == 0) {
+      Device* sel = ath_device_select(&handle, 3);
+      if (sel != dev) status = 3;
+    }
+    if (status == 0) {
+      ath_allocate(&handle, *dev, &tc);
+      ath_lock(&handle, *dev, &ta, 0);
+      ath_lock(&handle, *dev, &tb, 0);
+      ath_lock(&handle, *dev, &tc, 1);
+      ArgDesc args[5];
+      args[0] = ArgDesc{0, &ta, ArgDesc::TENSOR};
+      args[1] = ArgDesc{sizeof(float), &scaleA, ArgDesc::DATA};
+      args[2] = ArgDesc{0, &tb, ArgDesc::TENSOR};
+      args[3] = ArgDesc{sizeof(float), &scaleB, ArgDesc::DATA};
+      args[4] = ArgDesc{0, &tc, ArgDesc::TENSOR};
+      LaunchCommand cmd{"probe_fadd", 5, args, "fadd"};
+      evt = ath_launch(&handle, dev, nullptr, cmd);
+      if (evt == nullptr) status = 4;
+    }
+    if (status == 0) {
+      ath_release(&handle, *dev, &ta, evt);
+      ath_release(&handle, *dev, &tb, evt);
+      ath_release(&handle, *dev, &tc, evt);
+      Event* events[2] = {evt, nullptr}; // null entries are skipped
+      ath_barrier(2, events);
+      // output nodes: a host lock pulls the newest copy into RAM
+      for (auto [id, t] : {std::pair<uint64_t, TensorInfo*>{4, &tc}, {5, &ta}}) {
+        Device* host = ath_device_select(&handle, id);
+        ath_lock(&handle, *host, t, 0);
+        ath_load(&handle, id, t);
+        ath_release(&handle, *host, t, nullptr);
+      }
+    }
+  } // handle (allocator, host device) destroyed
+  return status;
 }
 
 } // extern "C"

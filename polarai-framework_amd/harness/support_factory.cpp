@@ -1,0 +1,34 @@
+// Construction helpers of the support library for callers that cannot name
+// its concrete classes.
+#include "devices.hpp"
+#include "support_routines.hpp"
+
+#include <cstddef>
+
+using namespace polar_harness_detail;
+
+extern "C" {
+
+BackendAllocator* polar_rt_support_allocator_create() { return new CoherentAllocator(); }
+
+void polar_rt_support_allocator_destroy(BackendAllocator* allocator) { delete allocator; }
+
+void polar_rt_support_register_device(BackendAllocator* allocator, Device* device) {
+  if (allocator == nullptr || device == nullptr)
+    fatalError(kFatalOther, "polar_rt_support_register_device: null argument");
+  allocator->registerDevice(*device);
+}
+
+Device* polar_rt_support_host_device_create() { return new HostDevice(); }
+
+void polar_rt_support_host_device_destroy(Device* device) { delete device; }
+
+void polar_rt_support_graph_handle_layout(uint64_t out[5]) {
+  out[0] = sizeof(GraphHandle);
+  out[1] = offsetof(GraphHandle, allocator);
+  out[2] = offsetof(GraphHandle, devices);
+  out[3] = offsetof(GraphHandle, mLoaders);
+  out[4] = offsetof(GraphHandle, isHostNode);
+}
+
+} // extern "C"

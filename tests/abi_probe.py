@@ -28,7 +28,29 @@ def load():
     lib.ref_allocator_and_copy.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t]
     lib.ref_launch_fadd.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64,
                                     C.c_uint64, C.c_float, C.c_float]
+    lib.ref_graph_handle_layout.argtypes = [C.POINTER(C.c_uint64)]
+    lib.ref_support_evaluate.argtypes = [C.c_void_p, C.c_uint64, C.c_void_p, C.c_void_p,
+                                         C.c_float, C.c_float, C.c_void_p, C.c_void_p]
     return lib
+
+
+def graph_handle_layouts(lib):
+    """(layout per the reference's GraphHandle.hpp, layout the support library was built with)"""
+    out = (C.c_uint64 * 10)()
+    lib.ref_graph_handle_layout(out)
+    return list(out[:5]), list(out[5:])
+
+
+def support_evaluate(lib, device_ptr, a, b, scale_a, scale_b):
+    """Two input nodes, one fadd node, barrier and host reads through the support
+    library's ath_* on a reference-declared GraphHandle.  Returns (rc, sum, a_back)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    total = np.full_like(a, np.nan)
+    a_back = np.full_like(a, np.nan)
+    rc = lib.ref_support_evaluate(device_ptr, a.size, a.ctypes.data, b.ctypes.data, scale_a, scale_b,
+                                  total.ctypes.data, a_back.ctypes.data)
+    return rc, total, a_back
 
 
 def struct_layout(lib):

@@ -48,6 +48,54 @@ def _exercise(h, expect_result):
 
 
 @needs_probe
+def test_graph_handle_layout_matches_the_reference_header():
+    reference, ours = abi_probe.graph_handle_layouts(abi_probe.load())
+    assert reference == ours and reference[1] == 0
+
+
+def _support_library_evaluate(h, expect_result):
+    """The support library (libpolar_rt_support_static.a, linked into the probe) driven
+    by a caller that declares GraphHandle, Device, Event and the launch structs from the
+    reference's headers."""
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(4099).astype(np.float32)
+    b = rng.standard_normal(4099).astype(np.float32)
+    rc, total, a_back = abi_probe.support_evaluate(abi_probe.load(), h.raw_device(), a, b, 0.25, -1.5)
+    assert rc == 0, f"support-library step {rc}"
+    assert np.array_equal(a_back, a)           # RAM copy intact after the device's READ lock
+    if expect_result:
+        assert np.array_equal(total, np.float32(0.25) * a + np.float32(-1.5) * b)
+
+
+def test_support_library_archive_defines_its_interface():
+    """libpolar_rt_support_static.a defines every function include/polar_rt_support.hpp declares."""
+    import os, re, subprocess
+    from polarai_framework_amd import PACKAGE_DIR as PKG_DIR
+    root = os.path.dirname(PKG_DIR)
+    header = open(os.path.join(root, "include", "polar_rt_support.hpp")).read()
+    declared = set(re.findall(r"\b(ath_\w+|polar_rt_support_\w+)\s*\(", header))
+    assert {"ath_allocate", "ath_release", "ath_lock", "ath_device_select", "ath_barrier", "ath_launch",
+            "ath_load"} <= declared
+    nm = subprocess.run(["nm", "-g", "--defined-only", os.path.join(PKG_DIR, "libpolar_rt_support_static.a")],
+                        check=True, capture_output=True, text=True).stdout
+    defined = set(re.findall(r" T (\w+)", nm))
+    assert declared <= defined, declared - defined
+
+
+@needs_probe
+def test_support_library_with_mock_device_and_reference_graph_handle():
+    with harness.Harness(plugin=None) as h:
+        _support_library_evaluate(h, expect_result=False)
+
+
+@needs_probe
+@pytest.mark.gpu
+def test_support_library_with_hip_plugin_and_reference_graph_handle():
+    with harness.Harness(plugin=LIB_PLUGIN) as h:
+        _support_library_evaluate(h, expect_result=True)
+
+
+@needs_probe
 def test_mock_device_through_reference_declarations():
     with harness.Harness(plugin=None) as h:
         _exercise(h, expect_result=False)
