@@ -176,6 +176,7 @@ def main():
     if not args.no_matmul:
         result["transpose"] = bench_transpose(dev, args)
         result["matmul"] = bench_matmul(dev, args)
+        result["next_builtins"] = bench_next_builtins(dev, da, n, args)
     da.free(); db.free()
     dev.close()
     dev = None
@@ -220,6 +221,51 @@ def bench_transpose(dev, args):
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(gbs / HBM_PEAK_GBS, 4),
                          "traffic": MEASURED_TRAFFIC_BYTES["ftranspose"]}}
+
+
+def bench_next_builtins(dev, dx, n, args):
+    """frelu / fsoftmax on the sweep's first input, fconv2d 3x3 and fpool 2x2/2 on
+    an 8192 x 8192 image: the builtins the reference has only as generated code."""
+    out = {}
+
+    def report(name, workload, ms, nbytes):
+        gbs = nbytes / (np.mean(ms) * 1e-3) / 1e9
+        log(f"{name:10s} {np.mean(ms) * 1e3:9.1f} us  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of HBM peak")
+        out[name] = {"workload": workload, "ms": round(float(np.mean(ms)), 5),
+                     "min_ms": round(float(np.min(ms)), 5), "GB/s": round(gbs, 1),
+                     "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(nbytes)}
+
+    dout = dev.empty(n)
+    ms = time_kernel(dev, lambda: dev.frelu(dx, dout), args.warmup, args.steps)
+    report("frelu", f"{n} elements, 1R+1W", ms, 8 * n)
+    # fsoftmax is three launches (partial sums, total, scale): timed with events around the call
+    for _ in range(args.warmup):
+        dev.fsoftmax(dx, dout)
+    dev.synchronize()
+    ms = []
+    for _ in range(args.steps):
+        e0 = dev.record(); dev.fsoftmax(dx, dout); e1 = dev.record()
+        e1.synchronize(); ms.append(e0.elapsed_ms(e1)); e0.release(); e1.release()
+    report("fsoftmax", f"{n} elements over the whole tensor, 2R+1W (sum pass, scale pass)", ms, 12 * n)
+    dout.free()
+
+    h = w = 8192
+    rng = np.random.default_rng(8)
+    img = rng.standard_normal((h, w), dtype=np.float32)
+    k = rng.standard_normal((3, 3), dtype=np.float32)
+    dimg, dk = dev.array(img), dev.array(k)
+    dconv = dev.empty((h - 2) * (w - 2))
+    ms = time_kernel(dev, lambda: dev.fconv2d(dimg, dk, dconv, h, w, 3, 3), args.warmup, args.steps)
+    report("fconv2d", f"{h}x{w} image, 3x3 kernel, valid correlation", ms, 4 * (h * w + (h - 2) * (w - 2)) + 36)
+    dconv.free()
+    dpool = dev.empty((h // 2) * (w // 2))
+    ms = time_kernel(dev, lambda: dev.fpool(dimg, dpool, h, w, (2, 2), (2, 2)), args.warmup, args.steps)
+    report("fpool", f"{h}x{w} image, max, window 2x2, stride 2x2", ms, 4 * (h * w + (h // 2) * (w // 2)))
+    got = dpool.download((h // 2, w // 2))[:8]
+    assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
+    for t in (dimg, dk, dpool):
+        t.free()
+    return out
 
 
 def bench_matmul(dev, args):

@@ -31,7 +31,8 @@ extern "C" {
 typedef struct polar_harness polar_harness;
 
 typedef struct polar_harness_arg {
-  int kind;       /* 0 = tensor (vaddr), 1 = fp32 scalar (scalar) */
+  int kind;       /* 0 = tensor (vaddr), 1 = fp32 scalar (scalar),
+                     2 = 64-bit integer scalar (value in vaddr) */
   uint64_t vaddr; /* virtual address returned by polar_harness_tensor */
   float scalar;
 } polar_harness_arg;

@@ -171,6 +171,39 @@ int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
                       const float* a, const float* b, float* c, uint64_t m,
                       uint64_t n, uint64_t k);
 
+/* ---- Builtins the reference specifies only as generated (MLIR) kernels ------
+ * Their hand-written runtimes have no entry for them; two of them cannot even
+ * be named there (ReLU and Softmax both answer "ftranspose" as their builtin
+ * name -- utils/dialects/include/PolarGraph/PolarGraphOps.td:462,501), so the
+ * plugin takes them under the names frelu / fsoftmax. */
+/* frelu: out[i] = in[i] > 0 ? in[i] : 0
+ * (utils/dialects/lib/PolarGraph/kernels/ReLUOp.cpp:35-44) */
+int polar_hip_frelu(polar_hip_device* dev, const float* in, float* out,
+                    uint64_t n);
+/* fsoftmax: out[i] = exp(in[i]) / sum_j exp(in[j]), the sum running over the
+ * WHOLE tensor, no max subtraction
+ * (utils/dialects/lib/PolarGraph/kernels/SoftmaxOp.cpp:38-65).  The sum is
+ * accumulated in fp64 in a fixed order and rounded to fp32 once. */
+int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out,
+                       uint64_t n);
+/* fconv2d: single-channel "valid" correlation, in is height x width, kernel
+ * kernelHeight x kernelWidth (odd sizes), out is (height-kernelHeight+1) x
+ * (width-kernelWidth+1); fp32 accumulation in tap order (a outer, b inner)
+ * (utils/dialects/lib/PolarGraph/kernels/Conv2DOp.cpp:35-84;
+ *  src/operation/internal/Conv2DOperationInternal.cpp:35-39). */
+int polar_hip_fconv2d(polar_hip_device* dev, const float* in,
+                      const float* kernel, float* out, uint64_t height,
+                      uint64_t width, uint64_t kernelHeight,
+                      uint64_t kernelWidth);
+/* fpool: max pooling, out[y,x] = max(-10e5, max over the window0 x window1
+ * block at (y*stride0, x*stride1)); out is ((height-window0)/stride0+1) x
+ * ((width-window1)/stride1+1)
+ * (utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:45-82;
+ *  src/operation/internal/Pool2DOperationInternal.cpp:37-41). */
+int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
+                    uint64_t height, uint64_t width, uint64_t window0,
+                    uint64_t window1, uint64_t stride0, uint64_t stride1);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,15 @@
  *                                    involution T(T(x)) = x and the identity
  *                                    matmul_t_f(A,B) == matmul_f_f(T(A),B).
  *
+ *   frelu, fsoftmax, fconv2d, fpool  one golden vector each from the reference's
+ *                                    integration tests, plus independent library
+ *                                    routines (numpy maximum, scipy softmax in
+ *                                    fp64, scipy correlate2d, reshape-max) on
+ *                                    random data.  fsoftmax at sizes where the
+ *                                    reference's sequential fp32 sum has lost
+ *                                    precision is checked against the fp64-
+ *                                    accumulated variant instead (see there).
+ *
  * Threads: polar_oracle_set_threads(n) selects how many host threads the
  * loops are split over (outermost index, static schedule).  n = 1 is the
  * faithful serial host-device loop; results do not depend on n.
@@ -242,6 +251,83 @@ void polar_oracle_fmatmul_f64acc(int transA, int transB, const float* A,
         acc += l * r;
       }
       C[i * (int64_t)N + j] = acc;
+    }
+  }
+}
+
+/* out[i] = in[i] > 0 ? in[i] : 0  (ordered compare: NaN gives 0)
+ * utils/dialects/lib/PolarGraph/kernels/ReLUOp.cpp:35-44 */
+void polar_oracle_frelu(const float* in, float* out, uint64_t n) {
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = in[i] > 0.0f ? in[i] : 0.0f;
+}
+
+/* out[i] = exp(in[i]) / sum_j exp(in[j]) over the WHOLE tensor (any rank, no
+ * max subtraction); the sum is an fp32 scalar accumulated in index order.
+ * utils/dialects/lib/PolarGraph/kernels/SoftmaxOp.cpp:38-65 (the reference
+ * recomputes the sum for every output element; the value is the same).
+ * Serial on purpose: the accumulation order is part of the definition. */
+void polar_oracle_fsoftmax(const float* in, float* out, uint64_t n) {
+  float total = 0.0f;
+  for (uint64_t j = 0; j < n; ++j) total = expf(in[j]) + total;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = expf(in[i]) / total;
+}
+
+/* Same definition with the sum accumulated in fp64 (then rounded to fp32
+ * once): what the reference's loop computes when no precision is lost, used
+ * for sizes where the sequential fp32 sum has drifted. */
+void polar_oracle_fsoftmax_f64sum(const float* in, float* out, uint64_t n) {
+  double total = 0.0;
+  for (uint64_t j = 0; j < n; ++j) total += (double)expf(in[j]);
+  const float t = (float)total;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t i = 0; i < (int64_t)n; ++i) out[i] = expf(in[i]) / t;
+}
+
+/* Single-channel "valid" 2-D correlation: in is H x W, kernel KH x KW, out is
+ * (H-KH+1) x (W-KW+1); out[y,x] = sum_a sum_b in[y+a, x+b] * kernel[a,b],
+ * fp32 accumulator starting at 0, a outer / b inner, product rounded before
+ * the add.
+ * utils/dialects/lib/PolarGraph/kernels/Conv2DOp.cpp:35-84 (loops run over
+ * [-K/2, K/2], i.e. 2*(K/2)+1 taps: only odd kernel sizes index inside the
+ * kernel tensor); output shape src/operation/internal/Conv2DOperationInternal.cpp:35-39. */
+void polar_oracle_fconv2d(const float* in, const float* kernel, float* out,
+                          uint64_t H, uint64_t W, uint64_t KH, uint64_t KW) {
+  const int64_t OH = (int64_t)H - (int64_t)KH + 1, OW = (int64_t)W - (int64_t)KW + 1;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t y = 0; y < OH; ++y) {
+    for (int64_t x = 0; x < OW; ++x) {
+      float acc = 0.0f;
+      for (int64_t a = 0; a < (int64_t)KH; ++a)
+        for (int64_t b = 0; b < (int64_t)KW; ++b) {
+          float prod = in[(y + a) * (int64_t)W + x + b] * kernel[a * (int64_t)KW + b];
+          acc = prod + acc;
+        }
+      out[y * OW + x] = acc;
+    }
+  }
+}
+
+/* Max pooling: out[y,x] = max(-10e5f, max_{a<win0, b<win1} in[y*s0+a, x*s1+b])
+ * (strict ordered greater-than, so NaN inputs are skipped), out is
+ * ((H-win0)/s0+1) x ((W-win1)/s1+1).
+ * utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:45-82; output shape
+ * src/operation/internal/Pool2DOperationInternal.cpp:37-41. */
+void polar_oracle_fpool(const float* in, float* out, uint64_t H, uint64_t W,
+                        uint64_t win0, uint64_t win1, uint64_t s0, uint64_t s1) {
+  const int64_t OH = ((int64_t)H - (int64_t)win0) / (int64_t)s0 + 1;
+  const int64_t OW = ((int64_t)W - (int64_t)win1) / (int64_t)s1 + 1;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+  for (int64_t y = 0; y < OH; ++y) {
+    for (int64_t x = 0; x < OW; ++x) {
+      float best = -10e5f;
+      for (int64_t a = 0; a < (int64_t)win0; ++a)
+        for (int64_t b = 0; b < (int64_t)win1; ++b) {
+          float v = in[(y * (int64_t)s0 + a) * (int64_t)W + x * (int64_t)s1 + b];
+          best = v > best ? v : best;
+        }
+      out[y * OW + x] = best;
     }
   }
 }

@@ -39,6 +39,11 @@ def lib():
         l.polar_oracle_fmatmul.argtypes = [C.c_int, C.c_int, _fp, _u64, _u64, _fp, _u64, _u64, _fp, _u64, _u64]
         l.polar_oracle_fmatmul_rows.argtypes = [C.c_int, C.c_int, _fp, _u64, _u64, _fp, _u64, _u64, _fp, _u64, _u64, _u64, _u64]
         l.polar_oracle_fmatmul_f64acc.argtypes = [C.c_int, C.c_int, _fp, _u64, _u64, _fp, _u64, _u64, _dp, _u64, _u64]
+        l.polar_oracle_frelu.argtypes = [_fp, _fp, _u64]
+        l.polar_oracle_fsoftmax.argtypes = [_fp, _fp, _u64]
+        l.polar_oracle_fsoftmax_f64sum.argtypes = [_fp, _fp, _u64]
+        l.polar_oracle_fconv2d.argtypes = [_fp, _fp, _fp, _u64, _u64, _u64, _u64]
+        l.polar_oracle_fpool.argtypes = [_fp, _fp, _u64, _u64, _u64, _u64, _u64, _u64]
         l.polar_oracle_record_bytes.argtypes = [C.c_int, _u64, C.POINTER(_u64)]
         l.polar_oracle_record_bytes.restype = _u64
         _lib = l
@@ -117,6 +122,41 @@ def ftranspose(x):
     assert x.ndim == 2
     out = np.empty((x.shape[1], x.shape[0]), dtype=np.float32)
     lib().polar_oracle_ftranspose(x.ravel(), out.ravel(), x.shape[0], x.shape[1])
+    return out
+
+
+def frelu(x):
+    x = _f32(x)
+    c = np.empty_like(x)
+    lib().polar_oracle_frelu(x.ravel(), c.ravel(), x.size)
+    return c
+
+
+def fsoftmax(x, f64sum=False):
+    """Softmax over the whole tensor; f64sum selects the fp64-accumulated sum."""
+    x = _f32(x)
+    c = np.empty_like(x)
+    fn = lib().polar_oracle_fsoftmax_f64sum if f64sum else lib().polar_oracle_fsoftmax
+    fn(x.ravel(), c.ravel(), x.size)
+    return c
+
+
+def fconv2d(x, kernel):
+    x, kernel = _f32(x), _f32(kernel)
+    assert x.ndim == 2 and kernel.ndim == 2
+    out = np.empty((x.shape[0] - kernel.shape[0] + 1, x.shape[1] - kernel.shape[1] + 1), dtype=np.float32)
+    lib().polar_oracle_fconv2d(x.ravel(), kernel.ravel(), out.ravel(), x.shape[0], x.shape[1],
+                               kernel.shape[0], kernel.shape[1])
+    return out
+
+
+def fpool(x, window, stride):
+    x = _f32(x)
+    assert x.ndim == 2
+    out = np.empty(((x.shape[0] - window[0]) // stride[0] + 1, (x.shape[1] - window[1]) // stride[1] + 1),
+                   dtype=np.float32)
+    lib().polar_oracle_fpool(x.ravel(), out.ravel(), x.shape[0], x.shape[1], window[0], window[1],
+                             stride[0], stride[1])
     return out
 
 

@@ -83,6 +83,10 @@ SIGNATURES = {
     "polar_hip_ffill": (_i, [_vp, _f, _vp, _u64]),
     "polar_hip_ftranspose": (_i, [_vp, _vp, _vp, _u64, _u64]),
     "polar_hip_fmatmul": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
+    "polar_hip_frelu": (_i, [_vp, _vp, _vp, _u64]),
+    "polar_hip_fsoftmax": (_i, [_vp, _vp, _vp, _u64]),
+    "polar_hip_fconv2d": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64]),
+    "polar_hip_fpool": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64, _u64]),
 }
 
 _lib = None
@@ -282,6 +286,20 @@ class Device:
 
     def ftranspose(self, src, dst, rows, cols):
         _check(self.lib, self.lib.polar_hip_ftranspose(self.handle, src.ptr, dst.ptr, rows, cols))
+
+    def frelu(self, x, out, n=None):
+        _check(self.lib, self.lib.polar_hip_frelu(self.handle, x.ptr, out.ptr, out.count if n is None else n))
+
+    def fsoftmax(self, x, out, n=None):
+        _check(self.lib, self.lib.polar_hip_fsoftmax(self.handle, x.ptr, out.ptr, out.count if n is None else n))
+
+    def fconv2d(self, x, kernel, out, height, width, kernel_height, kernel_width):
+        _check(self.lib, self.lib.polar_hip_fconv2d(self.handle, x.ptr, kernel.ptr, out.ptr, height, width,
+                                                    kernel_height, kernel_width))
+
+    def fpool(self, x, out, height, width, window, stride):
+        _check(self.lib, self.lib.polar_hip_fpool(self.handle, x.ptr, out.ptr, height, width,
+                                                  window[0], window[1], stride[0], stride[1]))
 
     def fmatmul(self, trans_a, trans_b, a, b, c, m, n, k):
         _check(self.lib, self.lib.polar_hip_fmatmul(

@@ -81,6 +81,19 @@ struct ScaleOp { // sycl/kernels/MulConcat.hpp:33-35 (g = gradient[0])
     return g * d;
   }
 };
+struct ReluOp { // utils/dialects/lib/PolarGraph/kernels/ReLUOp.cpp:35-44
+  static constexpr int NIN = 1;
+  __device__ __forceinline__ float apply(float x, float) const {
+    return x > 0.0f ? x : 0.0f; // ordered compare: NaN -> 0
+  }
+};
+struct SoftmaxScaleOp { // utils/dialects/lib/PolarGraph/kernels/SoftmaxOp.cpp:56-63
+  static constexpr int NIN = 1;
+  float total;
+  __device__ __forceinline__ float apply(float x, float) const {
+    return expf(x) / total;
+  }
+};
 struct CopyOp { // sycl/kernels/Copy.hpp:49-53
   static constexpr int NIN = 1;
   __device__ __forceinline__ float apply(float s, float) const { return s; }
@@ -111,6 +124,12 @@ template <typename Op> struct OpLoader {
 template <> struct OpLoader<ScaleOp> {
   __device__ static ScaleOp load(const ScaleOp&, const float* g) {
     return ScaleOp{g[0]};
+  }
+};
+
+template <> struct OpLoader<SoftmaxScaleOp> {
+  __device__ static SoftmaxScaleOp load(const SoftmaxScaleOp&, const float* t) {
+    return SoftmaxScaleOp{t[0]};
   }
 };
 
@@ -219,6 +238,56 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
   return POLAR_HIP_OK;
 }
 
+// ---- fsoftmax, first pass: total = sum exp(x) over the whole tensor ----------
+// Work-group g sums elements [g*kSumChunk, (g+1)*kSumChunk) into partial[g];
+// lanes and partials accumulate in fp64 and every order is fixed by the index,
+// so the result does not depend on scheduling.  Plain (temporal) loads: the
+// second pass reads the tensor again and should find it in cache if it fits.
+constexpr int kSumBlock = 256;
+constexpr uint64_t kSumChunk = 16384; // elements per work-group
+
+__device__ __forceinline__ double blockSum(double v, double* lds) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  if (lane == 0) lds[wave] = v;
+  __syncthreads();
+  double total = 0.0;
+  if (threadIdx.x == 0)
+    for (int w = 0; w < kSumBlock / 64; ++w) total += lds[w];
+  return total; // valid in thread 0
+}
+
+__global__ __launch_bounds__(kSumBlock) void expSumKernel(const float* x, uint64_t n,
+                                                          double* partial) {
+  __shared__ double lds[kSumBlock / 64];
+  const uint64_t begin = uint64_t(blockIdx.x) * kSumChunk;
+  const uint64_t end = begin + kSumChunk < n ? begin + kSumChunk : n;
+  double acc = 0.0;
+  if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0 && end - begin == kSumChunk) {
+    const v4f* x4 = reinterpret_cast<const v4f*>(x + begin);
+#pragma unroll 4
+    for (uint32_t i = threadIdx.x; i < kSumChunk / 4; i += kSumBlock) {
+      const v4f v = x4[i];
+      acc += (double(expf(v.x)) + double(expf(v.y))) + (double(expf(v.z)) + double(expf(v.w)));
+    }
+  } else {
+    for (uint64_t i = begin + threadIdx.x; i < end; i += kSumBlock) acc += double(expf(x[i]));
+  }
+  const double total = blockSum(acc, lds);
+  if (threadIdx.x == 0) partial[blockIdx.x] = total;
+}
+
+// one work-group: total of the partials, rounded to fp32 once
+__global__ __launch_bounds__(kSumBlock) void finishSumKernel(const double* partial,
+                                                             uint64_t count, float* total) {
+  __shared__ double lds[kSumBlock / 64];
+  double acc = 0.0;
+  for (uint64_t i = threadIdx.x; i < count; i += kSumBlock) acc += partial[i];
+  const double t = blockSum(acc, lds);
+  if (threadIdx.x == 0) total[0] = static_cast<float>(t);
+}
+
 } // namespace
 
 extern "C" {
@@ -282,6 +351,38 @@ int polar_hip_ffill(polar_hip_device* dev, float pattern, float* out,
   POLAR_HIP_REQUIRE(n == 0 || out, "null tensor");
   return launchEw<FillOp, 256, 1>(dev, FillOp{pattern}, nullptr, nullptr, nullptr,
                              out, n);
+}
+
+int polar_hip_frelu(polar_hip_device* dev, const float* in, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (in && out), "null tensor");
+  return launchEw<ReluOp>(dev, ReluOp{}, nullptr, in, nullptr, out, n);
+}
+
+int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (in && out), "null tensor");
+  if (n == 0) return POLAR_HIP_OK;
+  const uint64_t groups = (n + kSumChunk - 1) / kSumChunk;
+  POLAR_HIP_REQUIRE(groups < (1ull << 31), "tensor too large for one launch");
+  // workspace: one fp64 partial per work-group, then the fp32 total
+  void* workspace = nullptr;
+  int st = polar_hip_alloc(dev, groups * sizeof(double) + sizeof(float), &workspace);
+  if (st != POLAR_HIP_OK) return st;
+  double* partial = static_cast<double*>(workspace);
+  float* total = reinterpret_cast<float*>(partial + groups);
+  hipError_t e = hipSetDevice(dev->ordinal);
+  if (e == hipSuccess)
+    e = launchKernel(dev, expSumKernel, dim3(static_cast<unsigned>(groups)),
+                     dim3(kSumBlock), in, n, partial);
+  if (e == hipSuccess)
+    e = launchKernel(dev, finishSumKernel, dim3(1), dim3(kSumBlock),
+                     static_cast<const double*>(partial), groups, total);
+  if (e == hipSuccess)
+    st = launchEw<SoftmaxScaleOp>(dev, SoftmaxScaleOp{0.0f}, total, in, nullptr, out, n);
+  polar_hip_free(dev, workspace); // stream-ordered: reused only by later work
+  if (e != hipSuccess) return failHip(e, "fsoftmax launch");
+  return st;
 }
 
 } // extern "C"

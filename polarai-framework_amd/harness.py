@@ -154,6 +154,8 @@ class Harness:
         for i, a in enumerate(args):
             if isinstance(a, Tensor):
                 arr[i] = Arg(0, a.vaddr, 0.0)
+            elif isinstance(a, (int, np.integer)) and not isinstance(a, bool):
+                arr[i] = Arg(2, int(a), 0.0)     # integer attribute, passed as a 64-bit scalar
             else:
                 arr[i] = Arg(1, 0, float(a))
         self._ok(self.lib.polar_harness_node(self.h, kernel.encode(), len(args), arr, result_index),
@@ -176,7 +178,7 @@ class Harness:
     # builtin operations with the operand order of the launch lowering
     def fadd(self, a, sa, b, sb, out=None):
         out = out or self.tensor(*a.shape)
-        self.node("fadd", [a, sa, b, sb, out], 4)
+        self.node("fadd", [a, float(sa), b, float(sb), out], 4)
         return out
 
     def _binary(self, name, x, y, out=None, shape=None):
@@ -207,12 +209,33 @@ class Harness:
         return out
 
     def ffill(self, pattern, out):
-        self.node("ffill", [pattern, out], 1)
+        self.node("ffill", [float(pattern), out], 1)
         return out
 
     def ftranspose(self, a, out=None):
         out = out or self.tensor(a.shape[1], a.shape[0])
         self.node("ftranspose", [a, out], 1)
+        return out
+
+    def frelu(self, x, out=None):
+        out = out or self.tensor(*x.shape)
+        self.node("frelu", [x, out], 1)
+        return out
+
+    def fsoftmax(self, x, out=None):
+        out = out or self.tensor(*x.shape)
+        self.node("fsoftmax", [x, out], 1)
+        return out
+
+    def fconv2d(self, x, kernel, out=None):
+        out = out or self.tensor(x.shape[0] - kernel.shape[0] + 1, x.shape[1] - kernel.shape[1] + 1)
+        self.node("fconv2d", [x, kernel, out], 2)
+        return out
+
+    def fpool(self, x, window, stride, out=None):
+        out = out or self.tensor((x.shape[0] - window[0]) // stride[0] + 1,
+                                 (x.shape[1] - window[1]) // stride[1] + 1)
+        self.node("fpool", [x, out, int(window[0]), int(window[1]), int(stride[0]), int(stride[1])], 1)
         return out
 
     def fmatmul(self, ta, tb, a, b, out=None):

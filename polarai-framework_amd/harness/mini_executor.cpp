@@ -239,10 +239,14 @@ int polar_harness_run(polar_harness* h) {
       std::vector<TensorInfo> infos(n.args.size());
       std::vector<ArgDesc> descs(n.args.size());
       std::vector<float> scalars(n.args.size());
+      std::vector<int64_t> integers(n.args.size());
       for (size_t i = 0; i < n.args.size(); ++i) {
         if (n.args[i].kind == 0) {
           infos[i] = h->find(n.args[i].vaddr)->info();
           descs[i] = ArgDesc{0, &infos[i], ArgDesc::TENSOR};
+        } else if (n.args[i].kind == 2) {
+          integers[i] = static_cast<int64_t>(n.args[i].vaddr);
+          descs[i] = ArgDesc{sizeof(int64_t), &integers[i], ArgDesc::DATA};
         } else {
           scalars[i] = n.args[i].scalar;
           descs[i] = ArgDesc{sizeof(float), &scalars[i], ArgDesc::DATA};

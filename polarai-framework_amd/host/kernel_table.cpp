@@ -70,6 +70,32 @@ void needAtLeast(const LaunchCommand& cmd, const TensorArg& in, uint64_t n) {
           static_cast<unsigned long long>(n));
 }
 
+// Integer attribute passed as a scalar argument (4 or 8 bytes, signed).
+uint64_t countArg(const LaunchCommand& cmd, uint64_t i) {
+  if (i >= cmd.argsCount)
+    fatal("%s: argument %llu missing", cmd.nativeKernelName,
+          static_cast<unsigned long long>(i));
+  const ArgDesc& a = cmd.args[i];
+  if (a.type != ArgDesc::DATA || a.arg == nullptr)
+    fatal("%s: argument %llu must be a scalar", cmd.nativeKernelName,
+          static_cast<unsigned long long>(i));
+  int64_t v = 0;
+  if (a.size == 8) {
+    std::memcpy(&v, a.arg, 8);
+  } else if (a.size == 4) {
+    int32_t w;
+    std::memcpy(&w, a.arg, 4);
+    v = w;
+  } else {
+    fatal("%s: integer argument %llu has %llu bytes", cmd.nativeKernelName,
+          static_cast<unsigned long long>(i), static_cast<unsigned long long>(a.size));
+  }
+  if (v <= 0)
+    fatal("%s: integer argument %llu must be positive", cmd.nativeKernelName,
+          static_cast<unsigned long long>(i));
+  return static_cast<uint64_t>(v);
+}
+
 using Launcher = void (*)(HipDevice&, BackendAllocator&, LaunchCommand&);
 
 // [0]a T [1]scaleA D [2]b T [3]scaleB D [4]c T; range = c
@@ -105,6 +131,59 @@ void launchSigmoid(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
   checkStatus(polar_hip_fsigmoid(d.native(), d.resolve(al, in.record),
                                  d.resolve(al, out.record), out.count),
               "polar_hip_fsigmoid");
+}
+
+// [0]in T [1]out T (utils/dialects/include/PolarGraph/PolarGraphOps.td:447-466,
+// 486-505: operands (input, out))
+template <int (*Fn)(polar_hip_device*, const float*, float*, uint64_t)>
+void launchUnary(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
+  TensorArg in = tensorArg(cmd, 0), out = tensorArg(cmd, 1);
+  needAtLeast(cmd, in, out.count);
+  checkStatus(Fn(d.native(), d.resolve(al, in.record), d.resolve(al, out.record), out.count),
+              cmd.nativeKernelName);
+}
+
+// [0]input T [1]kernel T [2]out T, all 2-D
+// (utils/dialects/include/PolarGraph/PolarGraphOps.td:243-260)
+void launchConv2D(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
+  TensorArg in = tensorArg(cmd, 0), k = tensorArg(cmd, 1), out = tensorArg(cmd, 2);
+  if (in.info->dims != 2 || k.info->dims != 2 || out.info->dims != 2)
+    fatal("fconv2d: operands must be 2-D");
+  const uint64_t h = in.info->shape[0], w = in.info->shape[1];
+  const uint64_t kh = k.info->shape[0], kw = k.info->shape[1];
+  if (kh > h || kw > w || out.info->shape[0] != h - kh + 1 || out.info->shape[1] != w - kw + 1)
+    fatal("fconv2d: shapes do not agree: input %llux%llu, kernel %llux%llu, out %llux%llu",
+          (unsigned long long)h, (unsigned long long)w, (unsigned long long)kh,
+          (unsigned long long)kw, (unsigned long long)out.info->shape[0],
+          (unsigned long long)out.info->shape[1]);
+  checkStatus(polar_hip_fconv2d(d.native(), d.resolve(al, in.record), d.resolve(al, k.record),
+                                d.resolve(al, out.record), h, w, kh, kw),
+              "polar_hip_fconv2d");
+}
+
+// [0]input T [1]out T, then the op's attributes as integer scalars:
+// [2]window0 [3]window1 [4]stride0 [5]stride1.  Upstream keeps window and
+// stride as attributes of the graph op
+// (utils/dialects/include/PolarGraph/PolarGraphOps.td:405-445) and its launch
+// lowering forwards operands only, so a native fpool needs them appended.
+void launchPool(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
+  TensorArg in = tensorArg(cmd, 0), out = tensorArg(cmd, 1);
+  if (in.info->dims != 2 || out.info->dims != 2) fatal("fpool: operands must be 2-D");
+  if (cmd.argsCount < 6)
+    fatal("fpool: window and stride must follow the tensors as four integer scalars");
+  const uint64_t w0 = countArg(cmd, 2), w1 = countArg(cmd, 3);
+  const uint64_t s0 = countArg(cmd, 4), s1 = countArg(cmd, 5);
+  const uint64_t h = in.info->shape[0], w = in.info->shape[1];
+  if (w0 > h || w1 > w || out.info->shape[0] != (h - w0) / s0 + 1 ||
+      out.info->shape[1] != (w - w1) / s1 + 1)
+    fatal("fpool: shapes do not agree: input %llux%llu, window %llux%llu, stride %llux%llu, "
+          "out %llux%llu",
+          (unsigned long long)h, (unsigned long long)w, (unsigned long long)w0,
+          (unsigned long long)w1, (unsigned long long)s0, (unsigned long long)s1,
+          (unsigned long long)out.info->shape[0], (unsigned long long)out.info->shape[1]);
+  checkStatus(polar_hip_fpool(d.native(), d.resolve(al, in.record), d.resolve(al, out.record),
+                              h, w, w0, w1, s0, s1),
+              "polar_hip_fpool");
 }
 
 // [0]src T [1]dst T; the whole source is copied (sycl/kernels/Copy.hpp:38-53)
@@ -176,6 +255,10 @@ const TableEntry kTable[] = {
     {"fcopy", launchCopy},
     {"ffill", launchFill},
     {"ftranspose", launchTranspose},
+    {"frelu", launchUnary<polar_hip_frelu>},
+    {"fsoftmax", launchUnary<polar_hip_fsoftmax>},
+    {"fconv2d", launchConv2D},
+    {"fpool", launchPool},
     {"fmatmul_f_f", launchMatMul<false, false>},
     {"fmatmul_f_t", launchMatMul<false, true>},
     {"fmatmul_t_f", launchMatMul<true, false>},

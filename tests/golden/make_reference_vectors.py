@@ -14,6 +14,9 @@ independently of the oracle:
   * sigmoid and logloss are evaluated in fp64 with Python's math library and
     carry a tolerance (they go through exp/log whose last bit is
     implementation-defined).
+  * relu and pool expectations are the literals of the reference's tests; softmax
+    is evaluated in fp64 and checked against the reference's literals; conv2d
+    keeps the reference's literal with its 4-ulp comparison.
 Nothing here imports the oracle or the device library.
 """
 import json
@@ -95,6 +98,33 @@ e64 = float(eps)
 exp = [-(yy * math.log(pp + e64)) - (1 - yy) * math.log(1 - pp + e64) for pp, yy in zip(p, y)]
 cases.append(dict(kernel="flogloss", cite="tests/integration/operations/LogLossOperation.cpp:37-38",
                   predicted=p, truth=y, expected=exp, exact=False, rel_tol=1e-6))
+
+# tests/integration/operations/ReLUOperation.cpp:36-37 (expected is literal there)
+cases.append(dict(kernel="frelu", cite="tests/integration/operations/ReLUOperation.cpp:36-37",
+                  x=vec([-1, 1]), expected=vec([0, 1]), exact=True))
+
+# tests/integration/operations/SoftmaxOperation.cpp:36-39: shape {2,2}, softmax over the whole
+# tensor.  The reference compares with EXPECT_FLOAT_EQ (4 ulp) against the literals
+# {0.0320586, 0.08714432, 0.23688282, 0.64391426}; the expected values here are the fp64
+# evaluation of exp(x)/sum(exp), which those literals round.
+xs = [1.0, 2.0, 3.0, 4.0]
+den = sum(math.exp(v) for v in xs)
+exp = [math.exp(v) / den for v in xs]
+lit = [0.0320586, 0.08714432, 0.23688282, 0.64391426]
+assert all(abs(e - l) <= 4 * 2.0 ** -24 * l for e, l in zip(exp, lit))
+cases.append(dict(kernel="fsoftmax", cite="tests/integration/operations/SoftmaxOperation.cpp:36-39",
+                  x=xs, shape=[2, 2], expected=exp, exact=False, rel_tol=4 * 2.0 ** -23))
+
+# tests/integration/operations/Conv2DOperation.cpp:36-40: 4x4 ones, 3x3 kernel of 0.1,
+# expected {0.9 x4} under EXPECT_FLOAT_EQ (4 ulp; the nine-term fp32 sum is not exactly 0.9f)
+cases.append(dict(kernel="fconv2d", cite="tests/integration/operations/Conv2DOperation.cpp:36-40",
+                  x=vec([1] * 16), shape=[4, 4], weights=vec([0.1] * 9), kernel_shape=[3, 3],
+                  expected=[0.9] * 4, exact=False, rel_tol=4 * 2.0 ** -23))
+
+# tests/integration/operations/Pool2DOperation.cpp:36-49: 4x4 input, window {2,2}, stride {2,2}
+cases.append(dict(kernel="fpool", cite="tests/integration/operations/Pool2DOperation.cpp:36-49",
+                  x=vec([1, 0, 2, 3, 4, 6, 6, 8, 3, 1, 1, 0, 1, 2, 2, 4]), shape=[4, 4],
+                  window=[2, 2], stride=[2, 2], expected=vec([6, 8, 3, 4]), exact=True))
 
 out = os.path.join(os.path.dirname(os.path.abspath(__file__)), "reference_vectors.json")
 with open(out, "w") as fh:

@@ -71,6 +71,17 @@ def run_case_oracle(case):
         a = np.asarray(case["a"], dtype=np.float32).reshape(sa)
         b = np.asarray(case["b"], dtype=np.float32).reshape(sb)
         return o.fmatmul(case["transA"], case["transB"], a, b).ravel()
+    if kn == "frelu":
+        return o.frelu(case["x"])
+    if kn == "fsoftmax":
+        return o.fsoftmax(np.asarray(case["x"], dtype=np.float32).reshape(case["shape"])).ravel()
+    if kn == "fconv2d":
+        x = np.asarray(case["x"], dtype=np.float32).reshape(case["shape"])
+        w = np.asarray(case["weights"], dtype=np.float32).reshape(case["kernel_shape"])
+        return o.fconv2d(x, w).ravel()
+    if kn == "fpool":
+        x = np.asarray(case["x"], dtype=np.float32).reshape(case["shape"])
+        return o.fpool(x, case["window"], case["stride"]).ravel()
     raise KeyError(kn)
 
 
@@ -107,6 +118,20 @@ def run_case_device(dev, case):
             a, b = up(case["a"]), up(case["b"])
             c = dev.empty(case["m"] * case["n"]); bufs.append(c)
             dev.fmatmul(case["transA"], case["transB"], a, b, c, case["m"], case["n"], case["k"])
+        elif kn in ("frelu", "fsoftmax"):
+            x = up(case["x"])
+            c = dev.empty(x.count); bufs.append(c)
+            getattr(dev, kn)(x, c)
+        elif kn == "fconv2d":
+            x, w = up(case["x"]), up(case["weights"])
+            (h, wd), (kh, kw) = case["shape"], case["kernel_shape"]
+            c = dev.empty((h - kh + 1) * (wd - kw + 1)); bufs.append(c)
+            dev.fconv2d(x, w, c, h, wd, kh, kw)
+        elif kn == "fpool":
+            x = up(case["x"])
+            (h, wd), win, st = case["shape"], case["window"], case["stride"]
+            c = dev.empty(((h - win[0]) // st[0] + 1) * ((wd - win[1]) // st[1] + 1)); bufs.append(c)
+            dev.fpool(x, c, h, wd, win, st)
         else:
             raise KeyError(kn)
         return c.download()
@@ -130,7 +155,8 @@ def check_case(case, got):
 
 # ---- per-node checking of a kernel DAG run through the mini-executor ---------
 
-BIT_EXACT_KERNELS = {"fadd", "fmul", "fdivide", "fmulconcat", "fcopy", "ffill", "ftranspose"}
+BIT_EXACT_KERNELS = {"fadd", "fmul", "fdivide", "fmulconcat", "fcopy", "ffill", "ftranspose", "frelu",
+                     "fconv2d", "fpool"}
 
 
 def oracle_node(node, values):

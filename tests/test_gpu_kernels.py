@@ -286,3 +286,102 @@ def test_events_order_and_time(dev):
     assert e0.done() and e1.done()
     assert e0.elapsed_ms(e1) > 0
     e0.release(); e1.release(); x.free()
+
+
+# ---- relu / softmax / conv2d / pool ---------------------------------------------
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("misalign", [0, 3])
+def test_relu_bit_exact(dev, n, misalign):
+    _say("relu n=", n, "misalign=", misalign)
+    rng = np.random.default_rng(700 + n)
+    x = parity.normal(rng, n)
+    x[:: 7] = 0.0
+    if n > 5:
+        x[1], x[2], x[3] = np.nan, -np.inf, np.inf
+    dx, dout = dev.array(x, misalign), dev.empty(n, misalign)
+    dev.frelu(dx, dout)
+    assert np.array_equal(dout.download(), o.frelu(x))
+    dx.free(); dout.free()
+
+
+@pytest.mark.parametrize("n", [1, 4, 1000, 16384, 16385, 100003])
+def test_softmax_against_sequential_oracle(dev, n):
+    """Sizes at which the reference's sequential fp32 sum is still accurate:
+    1e-5 relative per element against it (tolerance of the parity contract)."""
+    _say("softmax n=", n)
+    rng = np.random.default_rng(800 + n)
+    x = parity.normal(rng, n, std=1.5)
+    for mis in (0, 1):
+        dx, dout = dev.array(x, mis), dev.empty(n, mis)
+        dev.fsoftmax(dx, dout)
+        got = dout.download()
+        assert parity.elementwise_rel_error(got, o.fsoftmax(x)) <= parity.ELEMENTWISE_REL
+        assert parity.elementwise_rel_error(got, o.fsoftmax(x, f64sum=True)) <= 2e-6
+        dx.free(); dout.free()
+
+
+def test_softmax_is_repeatable(dev):
+    n = 3_000_001
+    x = parity.normal(np.random.default_rng(9), n)
+    dx, d1, d2 = dev.array(x), dev.empty(n), dev.empty(n)
+    dev.fsoftmax(dx, d1)
+    dev.fsoftmax(dx, d2)
+    assert np.array_equal(d1.download(), d2.download())   # fixed summation order
+    for b in (dx, d1, d2):
+        b.free()
+
+
+CONV_SHAPES = [((4, 4), (3, 3)), ((3, 3), (3, 3)), ((37, 53), (3, 3)), ((300, 1000), (5, 5)),
+               ((129, 700), (7, 3)), ((64, 64), (1, 1)), ((1, 515), (1, 3)), ((515, 1), (3, 1)),
+               ((40, 300), (23, 23)), ((100, 2049), (3, 5)), ((33, 289), (9, 1))]
+
+
+@pytest.mark.parametrize("shape,kshape", CONV_SHAPES)
+def test_conv2d_bit_exact(dev, shape, kshape):
+    _say("conv2d", shape, kshape)
+    rng = np.random.default_rng(900 + shape[0] + kshape[1])
+    x, w = parity.normal(rng, shape), parity.normal(rng, kshape)
+    ref = o.fconv2d(x, w)
+    for mis in (0, 5):     # output base at and off a 128-byte line
+        dx, dw, dout = dev.array(x), dev.array(w), dev.empty(ref.size + 64, mis)
+        dev.ffill(-7.0, dout)
+        dev.fconv2d(dx, dw, dout, shape[0], shape[1], kshape[0], kshape[1])
+        got = dout.download()
+        assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+        assert np.all(got[ref.size:] == -7.0)          # nothing written past the end
+        for b in (dx, dw, dout):
+            b.free()
+
+
+def test_conv2d_rejects_even_kernels_and_oversized(dev):
+    from polarai_framework_amd import capi
+    dx, dw, dout = dev.empty(64), dev.empty(16), dev.empty(64)
+    with pytest.raises(capi.PolarHipError):
+        dev.fconv2d(dx, dw, dout, 8, 8, 2, 2)
+    with pytest.raises(capi.PolarHipError):
+        dev.fconv2d(dx, dw, dout, 2, 2, 3, 3)
+    for b in (dx, dw, dout):
+        b.free()
+
+
+POOL_CASES = [((4, 4), (2, 2), (2, 2)), ((100, 257), (2, 2), (2, 2)), ((101, 333), (3, 3), (2, 2)),
+              ((50, 50), (3, 2), (1, 3)), ((64, 64), (64, 64), (1, 1)), ((9, 1000), (1, 1), (1, 1)),
+              ((257, 1031), (2, 2), (2, 2)), ((16, 4100), (4, 4), (4, 4)), ((30, 30), (5, 5), (7, 7))]
+
+
+@pytest.mark.parametrize("shape,window,stride", POOL_CASES)
+def test_pool_bit_exact(dev, shape, window, stride):
+    _say("pool", shape, window, stride)
+    rng = np.random.default_rng(1000 + shape[1])
+    x = parity.normal(rng, shape)
+    x[0, 0] = -3e6                                     # below the -10e5 floor
+    ref = o.fpool(x, window, stride)
+    for mis in (0, 9):
+        dx, dout = dev.array(x), dev.empty(ref.size + 64, mis)
+        dev.ffill(-7.0, dout)
+        dev.fpool(dx, dout, shape[0], shape[1], window, stride)
+        got = dout.download()
+        assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+        assert np.all(got[ref.size:] == -7.0)
+        dx.free(); dout.free()

@@ -69,6 +69,18 @@ def _run_case(h, case):
         a, b = h.input(f32(case["a"], sa)), h.input(f32(case["b"], sb))
         h.end_cluster()
         out = h.fmatmul(case["transA"], case["transB"], a, b)
+    elif kn in ("frelu", "fsoftmax"):
+        x = h.input(f32(case["x"], case.get("shape", (len(case["x"]),))))
+        h.end_cluster()
+        out = getattr(h, kn)(x)
+    elif kn == "fconv2d":
+        x, w = h.input(f32(case["x"], case["shape"])), h.input(f32(case["weights"], case["kernel_shape"]))
+        h.end_cluster()
+        out = h.fconv2d(x, w)
+    elif kn == "fpool":
+        x = h.input(f32(case["x"], case["shape"]))
+        h.end_cluster()
+        out = h.fpool(x, case["window"], case["stride"])
     h.end_cluster()
     h.run()
     return h.read(out)

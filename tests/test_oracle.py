@@ -165,3 +165,90 @@ def test_record_bytes():
     assert o.record_bytes(1, [3]) == 24
     assert o.record_bytes(3, [2, 2, 2]) == 16
     assert o.record_bytes(2, []) == 4
+
+
+# ---- relu / softmax / conv2d / pool: independent library routines -------------
+
+def test_frelu_against_numpy_and_special_values():
+    rng = np.random.default_rng(31)
+    x = parity.normal(rng, 10007)
+    assert np.array_equal(o.frelu(x), np.maximum(x, np.float32(0)))
+    special = np.array([np.nan, -np.inf, np.inf, -0.0, 0.0, np.float32(1e-45)], dtype=np.float32)
+    got = o.frelu(special)
+    assert got[0] == 0 and got[1] == 0 and got[2] == np.inf and got[3] == 0 and got[4] == 0
+    assert got[5] == np.float32(1e-45)          # ordered greater-than: NaN -> 0, denormals kept
+
+
+def test_fsoftmax_against_fp64_library():
+    from scipy.special import softmax
+    rng = np.random.default_rng(32)
+    x = parity.normal(rng, (25, 40), std=2.0)
+    ref = softmax(x.astype(np.float64), axis=None)       # over the whole tensor, not per row
+    assert parity.elementwise_rel_error(o.fsoftmax(x), ref) <= 1e-5
+    assert parity.elementwise_rel_error(o.fsoftmax(x, f64sum=True), ref) <= 1e-6
+    assert abs(float(o.fsoftmax(x).astype(np.float64).sum()) - 1.0) < 1e-5
+    # a per-row softmax would differ grossly
+    assert parity.elementwise_rel_error(o.fsoftmax(x), softmax(x.astype(np.float64), axis=1)) > 0.5
+    # no max subtraction: large inputs overflow to inf/inf = nan exactly as exp(x)/sum does
+    with np.errstate(all="ignore"):
+        assert np.isnan(o.fsoftmax(np.array([100.0, 0.0], dtype=np.float32))[0])
+
+
+def test_fsoftmax_sum_is_sequential_fp32():
+    # 2^24 + 1 + 1 ... stagnates in fp32: with x = 0 everywhere the running sum stops at 2^24
+    n = (1 << 24) + 1000
+    x = np.zeros(n, dtype=np.float32)
+    assert o.fsoftmax(x)[0] == np.float32(1.0) / np.float32(1 << 24)
+    assert o.fsoftmax(x, f64sum=True)[0] == np.float32(1.0) / np.float32(n)
+
+
+@pytest.mark.parametrize("shape,kshape", [((4, 4), (3, 3)), ((17, 23), (5, 3)), ((9, 31), (1, 7)), ((12, 12), (11, 11))])
+def test_fconv2d_against_scipy_correlate(shape, kshape):
+    from scipy.signal import correlate2d
+    rng = np.random.default_rng(33)
+    # small integers: every product and partial sum is exact in fp32, so the
+    # result must EQUAL the library's (a flipped kernel, i.e. a true convolution,
+    # or a swapped index would not)
+    x = rng.integers(-8, 9, size=shape).astype(np.float32)
+    w = rng.integers(-4, 5, size=kshape).astype(np.float32)
+    ref = correlate2d(x.astype(np.float64), w.astype(np.float64), mode="valid")
+    assert np.array_equal(o.fconv2d(x, w), ref.astype(np.float32))
+    assert not np.array_equal(o.fconv2d(x, w[::-1, ::-1].copy()), ref.astype(np.float32)) or w.size == 1
+    xr, wr = parity.normal(rng, shape), parity.normal(rng, kshape)
+    ref = correlate2d(xr.astype(np.float64), wr.astype(np.float64), mode="valid")
+    assert parity.frobenius_rel_error(o.fconv2d(xr, wr), ref) <= 1e-6
+
+
+def test_fconv2d_accumulates_in_tap_order_unfused():
+    # taps chosen so that fp32 order matters: 1e8 + 1 - 1e8 is 0 in tap order, 1 if reordered
+    x = np.ones((1, 3), dtype=np.float32)
+    w = np.array([[1e8, 1.0, -1e8]], dtype=np.float32)
+    assert o.fconv2d(x, w)[0, 0] == 0.0
+    w2 = np.array([[1e8, -1e8, 1.0]], dtype=np.float32)
+    assert o.fconv2d(x, w2)[0, 0] == 1.0
+    # product rounded before the add (no fma): a*b + c with a*b inexact
+    a = np.float32(1 + 2 ** -12)
+    x3 = np.array([[a, 1.0]], dtype=np.float32)
+    w3 = np.array([[a, -(np.float32(a * a))]], dtype=np.float32)
+    assert o.fconv2d(x3, w3)[0, 0] == 0.0
+
+
+@pytest.mark.parametrize("shape,window,stride", [((4, 4), (2, 2), (2, 2)), ((9, 14), (3, 2), (3, 2)),
+                                                 ((10, 11), (3, 3), (2, 1)), ((7, 7), (7, 7), (1, 1)),
+                                                 ((8, 9), (1, 1), (3, 4))])
+def test_fpool_against_sliding_windows(shape, window, stride):
+    from numpy.lib.stride_tricks import sliding_window_view
+    rng = np.random.default_rng(34)
+    x = parity.normal(rng, shape)
+    ref = sliding_window_view(x, window)[::stride[0], ::stride[1]].max(axis=(2, 3))
+    got = o.fpool(x, window, stride)
+    assert got.shape == ref.shape == ((shape[0] - window[0]) // stride[0] + 1, (shape[1] - window[1]) // stride[1] + 1)
+    assert np.array_equal(got, ref)
+
+
+def test_fpool_floor_and_nan():
+    # the running maximum starts at -10e5: smaller inputs are clamped to it, NaN is skipped
+    x = np.array([[-2e6, -3e6], [np.nan, -5e6]], dtype=np.float32)
+    assert o.fpool(x, (2, 2), (2, 2))[0, 0] == np.float32(-10e5)
+    x[1, 1] = 7
+    assert o.fpool(x, (2, 2), (2, 2))[0, 0] == 7
