@@ -25,11 +25,25 @@ using namespace polar_hip_detail;
 
 namespace {
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 constexpr int kSegment = 256; // output columns per work-group = lanes
 constexpr int kLine = 32;     // floats per 128-byte line
-constexpr int kConvRows = 32; // output rows per fconv2d work-group
+constexpr int kConvRows = 16; // output rows per fconv2d work-group
 constexpr int kPoolRows = 8;  // output rows per fpool work-group
 constexpr uint32_t kMaxConvLds = 64 * 1024;
+
+// Work-group id -> tile index such that each XCD (ids equal modulo 8 share
+// one) works through a contiguous range of tiles: neighbouring tiles, which
+// share halo rows and columns, then meet in the same L2.  Returns false for
+// the padding groups at the end of the grid.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ bool tileOfGroup(uint32_t tiles, uint32_t* tile) {
+  const uint32_t perXcd = (tiles + kXcds - 1) / kXcds;
+  *tile = (blockIdx.x % kXcds) * perXcd + blockIdx.x / kXcds;
+  return blockIdx.x / kXcds < perXcd && *tile < tiles;
+}
+uint64_t paddedGrid(uint64_t tiles) { return (tiles + kXcds - 1) / kXcds * kXcds; }
 
 // columns the segments of output row y are shifted left by
 __device__ __forceinline__ uint32_t rowShift(uint32_t y, uint32_t ow, uint32_t basePhase) {
@@ -41,7 +55,7 @@ struct ConvArgs {
   const float* weights;
   float* out;
   uint32_t H, W, KH, KW, OH, OW;
-  uint32_t colTiles;
+  uint32_t colTiles, tiles;
   uint32_t outPhase; // (address of out / 4) mod 32
 };
 
@@ -50,7 +64,9 @@ template <int KH_, int KW_>
 __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   extern __shared__ float tile[];
   const uint32_t KH = KH_ ? KH_ : p.KH, KW = KW_ ? KW_ : p.KW;
-  const uint32_t ct = blockIdx.x % p.colTiles, rt = blockIdx.x / p.colTiles;
+  uint32_t tileIdx;
+  if (!tileOfGroup(p.tiles, &tileIdx)) return; // before any barrier
+  const uint32_t ct = tileIdx % p.colTiles, rt = tileIdx / p.colTiles;
   const uint32_t y0 = rt * kConvRows;
   const uint32_t rowsOut = p.OH - y0 < uint32_t(kConvRows) ? p.OH - y0 : uint32_t(kConvRows);
   const uint32_t rowsIn = rowsOut + KH - 1; // all inside the input: OH = H - KH + 1
@@ -58,27 +74,91 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   // input column held in tile column 0 (may be negative in the first segment)
   const int64_t x0 = int64_t(ct) * kSegment - (kLine - 1);
 
-  const uint32_t t = threadIdx.x, wave = t / 64, lane = t % 64;
-  for (uint32_t row = wave; row < rowsIn; row += kSegment / 64) {
-    const float* src = p.in + uint64_t(y0 + row) * p.W;
-    for (uint32_t col = lane; col < pitch; col += 64) {
-      const int64_t xi = x0 + col;
-      tile[row * pitch + col] = (xi >= 0 && xi < int64_t(p.W)) ? src[xi] : 0.0f;
+  // Stage the window: lane t takes elements t, t+256, ... of the window in
+  // row-major order.  pitch > 256, so stepping by 256 wraps to the next row at
+  // most once.
+  const uint32_t t = threadIdx.x;
+  bool staged = false;
+  if constexpr (KH_ != 0) {
+    // Full band of a constant-size kernel with the whole window inside the
+    // image: row and column of every element are compile-time constants plus
+    // one compare, nothing is predicated, and all loads are issued before the
+    // first LDS store.
+    constexpr uint32_t P = kSegment + (kLine - 1) + KW_ - 1;
+    constexpr uint32_t kRows = kConvRows + KH_ - 1;
+    constexpr uint32_t kTotal = kRows * P;
+    constexpr int kRounds = (kTotal + kSegment - 1) / kSegment;
+    if (x0 >= 0 && x0 + P <= int64_t(p.W) && rowsOut == uint32_t(kConvRows) &&
+        uint64_t(kRows) * p.W < (1u << 30)) {
+      const float* base = p.in + uint64_t(y0) * p.W + x0;
+      float v[kRounds];
+#pragma unroll
+      for (int u = 0; u < kRounds; ++u) {
+        const uint32_t k = uint32_t(u) * kSegment;
+        const uint32_t q = k / P, rem = k % P; // constants after unrolling
+        const bool wrap = t + rem >= P;
+        const uint32_t off = q * p.W + rem + t + (wrap ? p.W - P : 0u);
+        if (k + kSegment <= kTotal || k + t < kTotal) v[u] = base[off];
+      }
+#pragma unroll
+      for (int u = 0; u < kRounds; ++u) {
+        const uint32_t k = uint32_t(u) * kSegment;
+        if (k + kSegment <= kTotal || k + t < kTotal) tile[k + t] = v[u];
+      }
+      staged = true;
+    }
+  }
+  if (!staged) {
+    const uint32_t total = rowsIn * pitch;
+    constexpr int kBatch = 8;
+    uint32_t col = t;                                      // column within the window row
+    const float* src = p.in + uint64_t(y0) * p.W + x0 + t; // never dereferenced outside the image
+    for (uint32_t idx = t; idx < total; idx += kSegment * kBatch) {
+      float v[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int64_t xi = x0 + col;
+        const bool ok = idx + u * kSegment < total && xi >= 0 && xi < int64_t(p.W);
+        v[u] = ok ? *src : 0.0f;
+        col += kSegment;
+        src += kSegment;
+        if (col >= pitch) {
+          col -= pitch;
+          src += int64_t(p.W) - pitch;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u)
+        if (idx + u * kSegment < total) tile[idx + u * kSegment] = v[u];
     }
   }
   __syncthreads();
 
-  for (uint32_t r = 0; r < rowsOut; ++r) {
+  // A wave takes every fourth row of the band; a lane computes four adjacent
+  // outputs of it, so a tap row is read from LDS once for the four and the
+  // wave stores 1 KiB of contiguous, line-aligned output.
+  const uint32_t wave = t / 64, lane = t % 64;
+  for (uint32_t r = wave; r < rowsOut; r += kSegment / 64) {
     const uint32_t y = y0 + r;
     const uint32_t shift = rowShift(y, p.OW, p.outPhase);
-    const int64_t x = int64_t(ct) * kSegment - shift + t;
-    if (x >= 0 && x < int64_t(p.OW)) {
-      const float* win = tile + r * pitch + (t + (kLine - 1) - shift);
-      float acc = 0.0f;
-      for (uint32_t a = 0; a < KH; ++a)
-        for (uint32_t b = 0; b < KW; ++b)
-          acc = win[a * pitch + b] * p.weights[a * KW + b] + acc;
-      __builtin_nontemporal_store(acc, &p.out[uint64_t(y) * p.OW + uint64_t(x)]);
+    const int64_t x = int64_t(ct) * kSegment - shift + 4 * lane; // first of the four
+    if (x + 3 < 0 || x >= int64_t(p.OW)) continue;
+    const float* win = tile + r * pitch + (4 * lane + (kLine - 1) - shift);
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t a = 0; a < KH; ++a)
+      for (uint32_t b = 0; b < KW; ++b) {
+        const float wt = p.weights[a * KW + b];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + j] * wt + acc[j];
+      }
+    float* dst = p.out + uint64_t(y) * p.OW + x;
+    if (x >= 0 && x + 3 < int64_t(p.OW)) {
+      __builtin_nontemporal_store(v4f{acc[0], acc[1], acc[2], acc[3]},
+                                  reinterpret_cast<v4f*>(dst));
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (x + j >= 0 && x + j < int64_t(p.OW)) dst[j] = acc[j];
     }
   }
 }
@@ -102,12 +182,14 @@ struct PoolArgs {
   const float* in;
   float* out;
   uint32_t H, W, win0, win1, stride0, stride1, OH, OW;
-  uint32_t colTiles;
+  uint32_t colTiles, tiles;
   uint32_t outPhase;
 };
 
 __global__ __launch_bounds__(kSegment) void poolKernel(PoolArgs p) {
-  const uint32_t ct = blockIdx.x % p.colTiles, rt = blockIdx.x / p.colTiles;
+  uint32_t tileIdx;
+  if (!tileOfGroup(p.tiles, &tileIdx)) return;
+  const uint32_t ct = tileIdx % p.colTiles, rt = tileIdx / p.colTiles;
   const uint32_t y0 = rt * kPoolRows;
   const uint32_t rows = p.OH - y0 < uint32_t(kPoolRows) ? p.OH - y0 : uint32_t(kPoolRows);
   for (uint32_t r = 0; r < rows; ++r) {
@@ -170,8 +252,10 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in, const float* kerne
   const uint64_t ldsBytes = uint64_t(kConvRows + p.KH - 1) *
                             (kSegment + (kLine - 1) + p.KW - 1) * sizeof(float);
   if (ldsBytes <= kMaxConvLds) {
-    const uint64_t grid = uint64_t(p.colTiles) * ((p.OH + kConvRows - 1) / kConvRows);
-    POLAR_HIP_REQUIRE(grid < (1ull << 31), "tensor too large for one launch");
+    const uint64_t tiles = uint64_t(p.colTiles) * ((p.OH + kConvRows - 1) / kConvRows);
+    POLAR_HIP_REQUIRE(tiles < (1ull << 31) - kXcds, "tensor too large for one launch");
+    p.tiles = static_cast<uint32_t>(tiles);
+    const uint64_t grid = paddedGrid(tiles);
     auto fn = p.KH == 3 && p.KW == 3   ? conv2dKernel<3, 3>
               : p.KH == 5 && p.KW == 5 ? conv2dKernel<5, 5>
                                        : conv2dKernel<0, 0>;
@@ -180,6 +264,7 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in, const float* kerne
   } else {
     const uint64_t grid = uint64_t(p.colTiles) * p.OH;
     POLAR_HIP_REQUIRE(grid < (1ull << 31), "tensor too large for one launch");
+    p.tiles = static_cast<uint32_t>(grid);
     POLAR_HIP_TRY(launchKernel(dev, conv2dDirectKernel,
                                dim3(static_cast<unsigned>(grid)), dim3(kSegment), p));
   }
@@ -212,8 +297,10 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
   p.OW = (p.W - p.win1) / p.stride1 + 1;
   p.colTiles = (p.OW + (kLine - 1) + kSegment - 1) / kSegment;
   p.outPhase = phaseOf(out);
-  const uint64_t grid = uint64_t(p.colTiles) * ((p.OH + kPoolRows - 1) / kPoolRows);
-  POLAR_HIP_REQUIRE(grid < (1ull << 31), "tensor too large for one launch");
+  const uint64_t tiles = uint64_t(p.colTiles) * ((p.OH + kPoolRows - 1) / kPoolRows);
+  POLAR_HIP_REQUIRE(tiles < (1ull << 31) - kXcds, "tensor too large for one launch");
+  p.tiles = static_cast<uint32_t>(tiles);
+  const uint64_t grid = paddedGrid(tiles);
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   POLAR_HIP_TRY(launchKernel(dev, poolKernel, dim3(static_cast<unsigned>(grid)),
                              dim3(kSegment), p));

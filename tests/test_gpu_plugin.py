@@ -230,8 +230,33 @@ def _dies(code):
 
 def test_unknown_kernel_name_is_fatal():
     r = _dies("a = h.input(np.ones(4, dtype=np.float32)); h.end_cluster();"
-              "h.node('frelu', [a, h.tensor(4)], 1); h.end_cluster(); h.run()")
-    assert r.returncode != 0 and "no native kernel 'frelu'" in r.stderr
+              "h.node('fgelu', [a, h.tensor(4)], 1); h.end_cluster(); h.run()")
+    assert r.returncode != 0 and "no native kernel 'fgelu'" in r.stderr
+
+
+def test_pool_without_window_and_stride_is_fatal():
+    # upstream's lowering forwards operands only; a native fpool needs the attributes appended
+    r = _dies("a = h.input(np.ones((4, 4), dtype=np.float32)); h.end_cluster();"
+              "h.node('fpool', [a, h.tensor(2, 2)], 1); h.end_cluster(); h.run()")
+    assert r.returncode != 0 and "window and stride" in r.stderr
+
+
+def test_next_builtins_through_plugin(h):
+    rng = np.random.default_rng(52)
+    x = parity.normal(rng, (70, 300))
+    k = parity.normal(rng, (3, 3))
+    X, K = h.input(x), h.input(k)
+    h.end_cluster()
+    r = h.frelu(X)
+    s = h.fsoftmax(X)
+    c = h.fconv2d(X, K)
+    pl = h.fpool(X, (2, 3), (2, 2))
+    h.end_cluster()
+    h.run()
+    assert np.array_equal(h.read(r), o.frelu(x))
+    assert parity.elementwise_rel_error(h.read(s), o.fsoftmax(x)) <= parity.ELEMENTWISE_REL
+    assert np.array_equal(h.read(c), o.fconv2d(x, k))
+    assert np.array_equal(h.read(pl), o.fpool(x, (2, 3), (2, 2)))
 
 
 def test_mismatched_matmul_shapes_are_fatal():
