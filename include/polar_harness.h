@@ -74,6 +74,19 @@ int polar_harness_input(polar_harness* h, uint64_t vaddr, const float* data);
 int polar_harness_node(polar_harness* h, const char* native_kernel_name,
                        uint32_t nargs, const polar_harness_arg* args,
                        uint32_t result_index);
+/* Append a compute node whose kernel comes from the selected program: it is
+ * launched under jit_kernel_name with an empty native kernel name. */
+int polar_harness_jit_node(polar_harness* h, const char* jit_kernel_name,
+                           uint32_t nargs, const polar_harness_arg* args,
+                           uint32_t result_index);
+/* Hand the device one compiled program, as the executor does after compiling a
+ * graph (Device::selectBinary).  program_type is ProgramDesc::Type (0 PTX,
+ * 1 SPIRV_SHADER, 2 HSACO); geometry holds globalX,Y,Z,localX,Y,Z per kernel. */
+int polar_harness_select_binary(polar_harness* h, int program_type,
+                                const char* target, const void* image,
+                                uint64_t bytes, uint32_t kernel_count,
+                                const char* const* kernel_names,
+                                const uint64_t* geometry);
 /* Close the current cluster: a barrier over its launch events follows it. */
 int polar_harness_end_cluster(polar_harness* h);
 /* Drop all nodes (tensors and their contents stay). */

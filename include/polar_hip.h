@@ -171,6 +171,24 @@ int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
                       const float* a, const float* b, float* c, uint64_t m,
                       uint64_t n, uint64_t k);
 
+/* ---- Code objects compiled elsewhere (the framework's JIT) --------------------
+ * Counterpart of the module handling in the reference's CUDA runtime
+ * (src/backend/generic/runtime/cuda/CudaDevice.cpp:39-61 link/load,
+ *  :98-109 cuModuleGetFunction + cuLaunchKernel): load an AMDGPU code object
+ * (HSACO or an offload bundle holding a gfx950 image) and launch a kernel of
+ * it by name on the device's stream.  params[i] points at the i-th kernel
+ * parameter, as for cuLaunchKernel; grid counts work-groups. */
+typedef struct polar_hip_module polar_hip_module;
+int polar_hip_module_load(polar_hip_device* dev, const void* image,
+                          uint64_t bytes, polar_hip_module** out);
+int polar_hip_module_unload(polar_hip_device* dev, polar_hip_module* module);
+/* *found = 1 if the module defines a kernel of that name, else 0. */
+int polar_hip_module_has_kernel(polar_hip_module* module, const char* name,
+                                int* found);
+int polar_hip_module_launch(polar_hip_device* dev, polar_hip_module* module,
+                            const char* name, const uint32_t grid[3],
+                            const uint32_t block[3], void** params);
+
 /* ---- Builtins the reference specifies only as generated (MLIR) kernels ------
  * Their hand-written runtimes have no entry for them; two of them cannot even
  * be named there (ReLU and Softmax both answer "ftranspose" as their builtin

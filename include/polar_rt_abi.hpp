@@ -116,7 +116,10 @@ struct KernelDesc {
   size_t localX, localY, localZ;
 };
 struct ProgramDesc {
-  enum class Type { PTX, SPIRV_SHADER };
+  // PTX and SPIRV_SHADER are upstream's; HSACO (an AMDGPU code object, or an
+  // offload bundle holding one) is the value a HIP code generator would add --
+  // this runtime loads programs of that type in selectBinary.
+  enum class Type { PTX, SPIRV_SHADER, HSACO };
   Type type;
   std::string target;
   std::vector<char> data;

@@ -83,6 +83,11 @@ SIGNATURES = {
     "polar_hip_ffill": (_i, [_vp, _f, _vp, _u64]),
     "polar_hip_ftranspose": (_i, [_vp, _vp, _vp, _u64, _u64]),
     "polar_hip_fmatmul": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
+    "polar_hip_module_load": (_i, [_vp, _vp, _u64, C.POINTER(_vp)]),
+    "polar_hip_module_unload": (_i, [_vp, _vp]),
+    "polar_hip_module_has_kernel": (_i, [_vp, C.c_char_p, C.POINTER(_i)]),
+    "polar_hip_module_launch": (_i, [_vp, _vp, C.c_char_p, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                                     C.POINTER(_vp)]),
     "polar_hip_frelu": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fsoftmax": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fconv2d": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64]),

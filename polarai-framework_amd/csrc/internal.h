@@ -9,7 +9,9 @@
 #include <cstdarg>
 #include <cstdint>
 #include <map>
+#include <memory>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -42,6 +44,14 @@ struct polar_hip_device {
   polar_hip_event* timeStart = nullptr;
   polar_hip_event* timeStop = nullptr;
 
+};
+
+struct polar_hip_module {
+  polar_hip_device* dev = nullptr;
+  hipModule_t module = nullptr;
+  std::vector<char> image;
+  std::mutex mu;
+  std::unordered_map<std::string, hipFunction_t> functions; // null = not in the module
 };
 
 namespace polar_hip_detail {

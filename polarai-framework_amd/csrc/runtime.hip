@@ -386,4 +386,69 @@ int polar_hip_event_release(polar_hip_event* evt) {
   return POLAR_HIP_OK;
 }
 
+// ---- code objects -------------------------------------------------------------
+
+int polar_hip_module_load(polar_hip_device* dev, const void* image, uint64_t bytes,
+                          polar_hip_module** out) {
+  POLAR_HIP_REQUIRE(dev && image && out, "null argument");
+  POLAR_HIP_REQUIRE(bytes >= 4, "code object is empty");
+  *out = nullptr;
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  // the loader parses the image in place: keep a copy alive with the module
+  auto m = std::make_unique<polar_hip_module>();
+  m->dev = dev;
+  m->image.assign(static_cast<const char*>(image), static_cast<const char*>(image) + bytes);
+  POLAR_HIP_TRY(hipModuleLoadData(&m->module, m->image.data()));
+  *out = m.release();
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_module_unload(polar_hip_device* dev, polar_hip_module* module) {
+  POLAR_HIP_REQUIRE(dev && module && module->dev == dev, "module does not belong to this device");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(hipStreamSynchronize(dev->stream)); // its kernels may still run
+  hipError_t e = hipModuleUnload(module->module);
+  delete module;
+  if (e != hipSuccess) return failHip(e, "hipModuleUnload");
+  return POLAR_HIP_OK;
+}
+
+static hipFunction_t findKernel(polar_hip_module* module, const char* name) {
+  std::lock_guard<std::mutex> g(module->mu);
+  auto it = module->functions.find(name);
+  if (it != module->functions.end()) return it->second;
+  hipFunction_t fn = nullptr;
+  if (hipModuleGetFunction(&fn, module->module, name) != hipSuccess) {
+    (void)hipGetLastError(); // a missing name is an answer, not a sticky error
+    fn = nullptr;
+  }
+  module->functions.emplace(name, fn);
+  return fn;
+}
+
+int polar_hip_module_has_kernel(polar_hip_module* module, const char* name, int* found) {
+  POLAR_HIP_REQUIRE(module && name && found, "null argument");
+  POLAR_HIP_TRY(hipSetDevice(module->dev->ordinal));
+  *found = findKernel(module, name) != nullptr;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_module_launch(polar_hip_device* dev, polar_hip_module* module, const char* name,
+                            const uint32_t grid[3], const uint32_t block[3], void** params) {
+  POLAR_HIP_REQUIRE(dev && module && name && grid && block, "null argument");
+  POLAR_HIP_REQUIRE(module->dev == dev, "module does not belong to this device");
+  POLAR_HIP_REQUIRE(grid[0] >= 1 && grid[1] >= 1 && grid[2] >= 1 && block[0] >= 1 &&
+                        block[1] >= 1 && block[2] >= 1,
+                    "empty launch geometry");
+  POLAR_HIP_REQUIRE(uint64_t(block[0]) * block[1] * block[2] <= 1024,
+                    "more than 1024 lanes per work-group");
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  hipFunction_t fn = findKernel(module, name);
+  if (fn == nullptr)
+    return fail(POLAR_HIP_ERR_INVALID, "polar_hip_module_launch: no kernel '%s' in the module", name);
+  POLAR_HIP_TRY(hipModuleLaunchKernel(fn, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                      0, dev->stream, params, nullptr));
+  return POLAR_HIP_OK;
+}
+
 } // extern "C"

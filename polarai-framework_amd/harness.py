@@ -38,6 +38,9 @@ SIGNATURES = {
     "polar_harness_tensor": (_u64, [_vp, _u64, C.POINTER(_u64)]),
     "polar_harness_input": (_i, [_vp, _u64, _vp]),
     "polar_harness_node": (_i, [_vp, C.c_char_p, C.c_uint32, C.POINTER(Arg), C.c_uint32]),
+    "polar_harness_jit_node": (_i, [_vp, C.c_char_p, C.c_uint32, C.POINTER(Arg), C.c_uint32]),
+    "polar_harness_select_binary": (_i, [_vp, _i, C.c_char_p, C.c_char_p, _u64, C.c_uint32,
+                                         C.POINTER(C.c_char_p), C.POINTER(_u64)]),
     "polar_harness_end_cluster": (_i, [_vp]),
     "polar_harness_clear_program": (_i, [_vp]),
     "polar_harness_run": (_i, [_vp]),
@@ -149,7 +152,7 @@ class Harness:
         self._ok(self.lib.polar_harness_input(self.h, t.vaddr, None), "holder")
         return t
 
-    def node(self, kernel, args, result_index):
+    def _args(self, args):
         arr = (Arg * len(args))()
         for i, a in enumerate(args):
             if isinstance(a, Tensor):
@@ -158,8 +161,25 @@ class Harness:
                 arr[i] = Arg(2, int(a), 0.0)     # integer attribute, passed as a 64-bit scalar
             else:
                 arr[i] = Arg(1, 0, float(a))
+        return arr
+
+    def node(self, kernel, args, result_index):
+        arr = self._args(args)
         self._ok(self.lib.polar_harness_node(self.h, kernel.encode(), len(args), arr, result_index),
                  f"node {kernel}")
+
+    def jit_node(self, jit_kernel_name, args, result_index):
+        """A node whose kernel comes from the selected program (no native kernel name)."""
+        arr = self._args(args)
+        self._ok(self.lib.polar_harness_jit_node(self.h, jit_kernel_name.encode(), len(args), arr, result_index),
+                 f"jit node {jit_kernel_name}")
+
+    def select_binary(self, image, kernels, program_type=2, target="gfx950"):
+        """kernels: {name: (globalX, globalY, globalZ, localX, localY, localZ)}"""
+        names = (C.c_char_p * len(kernels))(*[k.encode() for k in kernels])
+        geo = (C.c_uint64 * (6 * len(kernels)))(*[int(v) for g in kernels.values() for v in g])
+        self._ok(self.lib.polar_harness_select_binary(self.h, program_type, target.encode(), image, len(image),
+                                                      len(kernels), names, geo), "select_binary")
 
     def end_cluster(self):
         self._ok(self.lib.polar_harness_end_cluster(self.h), "end_cluster")

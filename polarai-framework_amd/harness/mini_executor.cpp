@@ -40,7 +40,8 @@ struct TensorDecl {
 struct NodeDecl {
   uint64_t id;
   bool isInput;
-  std::string kernel;
+  std::string kernel;   // native kernel name ("" for a kernel of the selected program)
+  std::string jitName;  // name of the generated kernel; derived from the node when empty
   std::vector<polar_harness_arg> args;
   uint32_t result;      // index into args (compute) ...
   uint64_t inputVaddr;  // ... or the tensor an input node fills
@@ -187,6 +188,34 @@ int polar_harness_node(polar_harness* h, const char* native_kernel_name, uint32_
   return 0;
 }
 
+int polar_harness_jit_node(polar_harness* h, const char* jit_kernel_name, uint32_t nargs,
+                           const polar_harness_arg* args, uint32_t result_index) {
+  if (jit_kernel_name == nullptr || jit_kernel_name[0] == 0) return -1;
+  if (polar_harness_node(h, "", nargs, args, result_index) != 0) return -1;
+  h->clusters.back().back().jitName = jit_kernel_name;
+  return 0;
+}
+
+// src/backend/generic/lib/ExecutorImpl.cpp:52-64: after a graph is compiled the
+// executor passes the generated programs to every device.
+int polar_harness_select_binary(polar_harness* h, int program_type, const char* target,
+                                const void* image, uint64_t bytes, uint32_t kernel_count,
+                                const char* const* kernel_names, const uint64_t* geometry) {
+  if (h == nullptr || image == nullptr || (kernel_count != 0 && (!kernel_names || !geometry)))
+    return -1;
+  auto program = std::make_shared<ProgramDesc>();
+  program->type = static_cast<ProgramDesc::Type>(program_type);
+  program->target = target ? target : "";
+  program->data.assign(static_cast<const char*>(image), static_cast<const char*>(image) + bytes);
+  for (uint32_t i = 0; i < kernel_count; ++i) {
+    const uint64_t* g = geometry + 6 * i;
+    program->kernels[kernel_names[i]] = KernelDesc{g[0], g[1], g[2], g[3], g[4], g[5]};
+  }
+  std::vector<std::shared_ptr<ProgramDesc>> programs{program};
+  h->device->selectBinary(programs);
+  return 0;
+}
+
 int polar_harness_end_cluster(polar_harness* h) {
   if (h == nullptr) return -1;
   h->clusters.emplace_back();
@@ -264,7 +293,8 @@ int polar_harness_run(polar_harness* h) {
         ath_lock(&gh, *dev, &infos[i], LockType::READ);
         readLocked.push_back(i);
       }
-      const std::string jitName = "node" + std::to_string(n.id) + "_" + n.kernel;
+      const std::string jitName =
+          n.jitName.empty() ? "node" + std::to_string(n.id) + "_" + n.kernel : n.jitName;
       LaunchCommand cmd{jitName.c_str(), descs.size(), descs.data(), n.kernel.c_str()};
       Event* evt = ath_launch(&gh, dev, nullptr, cmd);
       for (size_t i : readLocked) ath_release(&gh, *dev, &infos[i], evt);

@@ -22,6 +22,7 @@ HipDevice::HipDevice(int ordinal) {
 
 HipDevice::~HipDevice() {
   if (mDev) polar_hip_device_synchronize(mDev);
+  if (mModule != nullptr) polar_hip_module_unload(mDev, mModule);
   mIdleEvents.clear();
   mEvents.clear();    // returns native events to the device's pool
   mAllocator->detach(); // other owners may keep the layer; its blocks die here
@@ -78,13 +79,114 @@ Event* HipDevice::launch(BackendAllocator& allocator, LaunchCommand& cmd,
                          Event* blockingEvent) {
   if (blockingEvent != nullptr && blockingEvent->getDevice() != this)
     blockingEvent->wait();
-  if (cmd.nativeKernelName == nullptr)
-    fatal("launch of '%s' without a native kernel name",
-          cmd.kernelName ? cmd.kernelName : "?");
-  if (!dispatchNativeKernel(*this, allocator, cmd))
+  // Hand-written kernels first; a kernel of the selected code object otherwise.
+  const bool native = cmd.nativeKernelName != nullptr && cmd.nativeKernelName[0] != 0 &&
+                      dispatchNativeKernel(*this, allocator, cmd);
+  if (!native && !launchFromProgram(allocator, cmd)) {
+    if (cmd.nativeKernelName == nullptr || cmd.nativeKernelName[0] == 0)
+      fatal("launch of '%s' without a native kernel name, and no selected program defines it",
+            cmd.kernelName ? cmd.kernelName : "?");
     fatal("no native kernel '%s' (requested by '%s')", cmd.nativeKernelName,
           cmd.kernelName ? cmd.kernelName : "?");
+  }
   return newEvent();
+}
+
+// Keeps the first HSACO program whose target names this device's architecture
+// (or no target).  The reference's CUDA runtime does the same with the first
+// PTX program (src/backend/generic/runtime/cuda/CudaDevice.cpp:39-61); its SYCL
+// runtime ignores programs altogether (sycl/SYCLDevice.h:121-122).
+void HipDevice::selectBinary(std::vector<std::shared_ptr<ProgramDesc>>& programs) {
+  polar_hip_device_info info;
+  checkStatus(polar_hip_device_get_info(mDev, &info), "polar_hip_device_get_info");
+  std::string arch = info.arch;
+  arch = arch.substr(0, arch.find(':'));
+  for (auto& program : programs) {
+    if (program == nullptr || program->type != ProgramDesc::Type::HSACO) continue;
+    if (!program->target.empty() && program->target.compare(0, arch.size(), arch) != 0) continue;
+    if (mModule != nullptr) {
+      checkStatus(polar_hip_module_unload(mDev, mModule), "polar_hip_module_unload");
+      mModule = nullptr;
+    }
+    checkStatus(polar_hip_module_load(mDev, program->data.data(), program->data.size(), &mModule),
+                "polar_hip_module_load");
+    mProgram = program;
+    return;
+  }
+}
+
+// Launch cmd.kernelName from the selected program with the geometry recorded
+// for it.  Tensor arguments expand to a memref descriptor -- allocated
+// pointer, aligned pointer, offset, sizes, strides -- as the generated code
+// expects (cuda/CudaDevice.cpp:75-94; the strides there are zeros, here they
+// are the row-major strides of the dense tensor); scalars are passed through.
+bool HipDevice::launchFromProgram(BackendAllocator& allocator, LaunchCommand& cmd) {
+  if (mModule == nullptr || cmd.kernelName == nullptr) return false;
+  auto geometry = mProgram->kernels.find(cmd.kernelName);
+  if (geometry == mProgram->kernels.end()) return false;
+  int found = 0;
+  checkStatus(polar_hip_module_has_kernel(mModule, cmd.kernelName, &found),
+              "polar_hip_module_has_kernel");
+  if (!found) return false;
+
+  std::vector<void*> pointers;          // device pointers, two slots per tensor
+  std::vector<int64_t> integers;        // offsets, sizes, strides
+  std::vector<std::pair<int, size_t>> layout; // (0 pointer / 1 integer / 2 scalar, index)
+  uint64_t tensors = 0, words = 0;
+  for (uint64_t i = 0; i < cmd.argsCount; ++i)
+    if (cmd.args[i].type == ArgDesc::TENSOR) {
+      ++tensors;
+      words += 1 + 2 * static_cast<TensorInfo*>(cmd.args[i].arg)->dims;
+    }
+  pointers.reserve(2 * tensors); // addresses of the elements are taken below
+  integers.reserve(words);
+  for (uint64_t i = 0; i < cmd.argsCount; ++i) {
+    const ArgDesc& a = cmd.args[i];
+    if (a.arg == nullptr) fatal("%s: argument %llu is null", cmd.kernelName, (unsigned long long)i);
+    if (a.type != ArgDesc::TENSOR) {
+      layout.emplace_back(2, i);
+      continue;
+    }
+    auto* t = static_cast<TensorInfo*>(a.arg);
+    if (t->dataType != static_cast<int>(core::DataType::FLOAT))
+      fatal("%s: tensor %llu has data type %d; this runtime is fp32 only", cmd.kernelName,
+            (unsigned long long)t->virtAddr, t->dataType);
+    MemoryRecord record{static_cast<size_t>(t->virtAddr), 4};
+    for (uint64_t d = 0; d < t->dims; ++d) record.allocationSize *= t->shape[d];
+    float* ptr = resolve(allocator, record);
+    for (int k = 0; k < 2; ++k) {
+      layout.emplace_back(0, pointers.size());
+      pointers.push_back(ptr);
+    }
+    layout.emplace_back(1, integers.size());
+    integers.push_back(0); // offset
+    for (uint64_t d = 0; d < t->dims; ++d) {
+      layout.emplace_back(1, integers.size());
+      integers.push_back(static_cast<int64_t>(t->shape[d]));
+    }
+    const size_t firstStride = integers.size();
+    for (uint64_t d = 0; d < t->dims; ++d) {
+      layout.emplace_back(1, integers.size());
+      integers.push_back(1);
+    }
+    for (uint64_t d = t->dims; d-- > 1;)
+      integers[firstStride + d - 1] =
+          integers[firstStride + d] * static_cast<int64_t>(t->shape[d]);
+  }
+  std::vector<void*> params;
+  params.reserve(layout.size());
+  for (auto& [kind, index] : layout)
+    params.push_back(kind == 0   ? static_cast<void*>(&pointers[index])
+                     : kind == 1 ? static_cast<void*>(&integers[index])
+                                 : cmd.args[index].arg);
+  const KernelDesc& k = geometry->second;
+  const uint32_t grid[3] = {static_cast<uint32_t>(k.globalX), static_cast<uint32_t>(k.globalY),
+                            static_cast<uint32_t>(k.globalZ)};
+  const uint32_t block[3] = {static_cast<uint32_t>(k.localX), static_cast<uint32_t>(k.localY),
+                             static_cast<uint32_t>(k.localZ)};
+  checkStatus(polar_hip_module_launch(mDev, mModule, cmd.kernelName, grid, block, params.data()),
+              "polar_hip_module_launch");
+  return true;
 }
 
 void HipDevice::consumeEvent(Event* evt) {

@@ -117,15 +117,18 @@ public:
   Event* launch(BackendAllocator& allocator, LaunchCommand& cmd,
                 Event* blockingEvent) override;
   void consumeEvent(Event* evt) override;
-  void selectBinary(std::vector<std::shared_ptr<ProgramDesc>>&) override {}
+  void selectBinary(std::vector<std::shared_ptr<ProgramDesc>>& programs) override;
 
   polar_hip_device* native() const { return mDev; }
   float* resolve(BackendAllocator& allocator, const MemoryRecord& record);
 
 private:
   HipEvent* newEvent();
+  bool launchFromProgram(BackendAllocator& allocator, LaunchCommand& cmd);
 
   polar_hip_device* mDev = nullptr;
+  std::shared_ptr<ProgramDesc> mProgram; // selected code object (kernel geometry lives here)
+  polar_hip_module* mModule = nullptr;
   std::string mName;
   std::shared_ptr<HipPoolAllocator> mAllocator;
   std::mutex mEventMutex;

@@ -263,3 +263,64 @@ def test_mismatched_matmul_shapes_are_fatal():
     r = _dies("a = h.input(np.ones((4, 5), dtype=np.float32)); b = h.input(np.ones((6, 3), dtype=np.float32));"
               "h.end_cluster(); h.node('fmatmul_f_f', [a, b, h.tensor(4, 3)], 2); h.end_cluster(); h.run()")
     assert r.returncode != 0 and "shapes do not agree" in r.stderr
+
+
+# ---- kernels from a selected program (Device::selectBinary) ------------------------
+
+CODE_OBJECT = os.path.join(os.path.dirname(os.path.abspath(__file__)), "native", "build",
+                           "generated_kernels.hsaco")
+
+
+def _code_object():
+    assert os.path.exists(CODE_OBJECT), "tests/native/build/generated_kernels.hsaco missing: run __graft_entry__.build()"
+    with open(CODE_OBJECT, "rb") as fh:
+        return fh.read()
+
+
+def test_program_kernels_run_when_no_native_kernel_is_named(h):
+    """A code object handed over through selectBinary; nodes without a native
+    kernel name launch its kernels by their generated name, with tensors
+    expanded to memref descriptors and the recorded launch geometry."""
+    rng = np.random.default_rng(53)
+    n, rows, cols = 5000, 37, 130
+    x, y = parity.normal(rng, n), parity.normal(rng, n)
+    m, s = parity.normal(rng, (rows, cols)), parity.normal(rng, rows)
+    h.select_binary(_code_object(), {
+        "gen_axpy_1d": (8, 1, 1, 256, 1, 1),
+        "gen_row_scale_2d": ((cols + 63) // 64, (rows + 3) // 4, 1, 64, 4, 1)})
+    X, Y, M, S = h.input(x), h.input(y), h.input(m), h.input(s)
+    h.end_cluster()
+    out1 = h.tensor(n)
+    h.jit_node("gen_axpy_1d", [X, 0.5, Y, out1], 3)
+    out2 = h.tensor(rows, cols)
+    h.jit_node("gen_row_scale_2d", [M, S, out2], 2)
+    native = h.fmul(X, Y)                       # hand-written kernels keep working beside it
+    h.end_cluster()
+    chained = h.frelu(out1)                     # and consume a program kernel's result
+    h.end_cluster()
+    h.run()
+    ref1 = np.float32(0.5) * x + y
+    assert np.array_equal(h.read(out1), ref1)
+    assert np.array_equal(h.read(out2), m * s[:, None])
+    assert np.array_equal(h.read(native), o.fmul(x, y))
+    assert np.array_equal(h.read(chained), o.frelu(ref1))
+
+
+def test_program_of_another_type_or_target_is_not_selected():
+    _code_object()
+    r = _dies(f"img = open({CODE_OBJECT!r}, 'rb').read();"
+              "h.select_binary(img, {'gen_axpy_1d': (8, 1, 1, 256, 1, 1)}, program_type=0);"       # PTX
+              "h.select_binary(img, {'gen_axpy_1d': (8, 1, 1, 256, 1, 1)}, target='gfx90a');"
+              "a = h.input(np.ones(4, dtype=np.float32)); h.end_cluster();"
+              "h.jit_node('gen_axpy_1d', [a, 1.0, a, h.tensor(4)], 3); h.end_cluster(); h.run()")
+    assert r.returncode != 0 and "without a native kernel name" in r.stderr
+
+
+def test_native_kernel_wins_over_a_program_kernel_of_the_same_node(h):
+    h.select_binary(_code_object(), {"gen_axpy_1d": (8, 1, 1, 256, 1, 1)})
+    a = h.input(np.arange(8, dtype=np.float32))
+    h.end_cluster()
+    out = h.fadd(a, 2.0, a, 3.0)
+    h.end_cluster()
+    h.run()
+    assert np.array_equal(h.read(out), np.arange(8, dtype=np.float32) * 5)
