@@ -43,8 +43,9 @@ SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
 # (profiles/bench_kernels_pmc_traffic.md).  They cannot be measured from inside
 # this process, so they are constants of the committed kernels.
 MEASURED_TRAFFIC_BYTES = {
-    "fadd": 805166953, "fmul": 805157993, "fdivide": 805155989, "fsigmoid": 536769637,
-    "fcopy": 536870912, "ffill": 268482969, "ftranspose": 776973224, "fmatmul": 469770774,
+    "fadd": 804971090, "fmul": 804957950, "fdivide": 804973820, "fsigmoid": 536570873,
+    "fcopy": 536870912, "ffill": 268298771, "ftranspose": 703413924, "fmatmul": 469719808,
+    "frelu": 536692356, "fsoftmax": 805229623, "fconv2d": 537078775, "fpool": 335466015,
 }
 T_ROWS, T_COLS = 12345, 6789
 MM = 4096
@@ -233,7 +234,8 @@ def bench_next_builtins(dev, dx, n, args):
         log(f"{name:10s} {np.mean(ms) * 1e3:9.1f} us  {gbs:8.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}% of HBM peak")
         out[name] = {"workload": workload, "ms": round(float(np.mean(ms)), 5),
                      "min_ms": round(float(np.min(ms)), 5), "GB/s": round(gbs, 1),
-                     "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(nbytes)}
+                     "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(nbytes),
+                     "traffic": MEASURED_TRAFFIC_BYTES[name] if n == N_SWEEP else None}
 
     dout = dev.empty(n)
     ms = time_kernel(dev, lambda: dev.frelu(dx, dout), args.warmup, args.steps)

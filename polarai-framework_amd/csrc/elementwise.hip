@@ -240,11 +240,12 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
 
 // ---- fsoftmax, first pass: total = sum exp(x) over the whole tensor ----------
 // Work-group g sums elements [g*kSumChunk, (g+1)*kSumChunk) into partial[g];
-// lanes and partials accumulate in fp64 and every order is fixed by the index,
+// lanes and partials accumulate in fp64 (groups of four terms in fp32 first)
+// and every order is fixed by the index,
 // so the result does not depend on scheduling.  Plain (temporal) loads: the
 // second pass reads the tensor again and should find it in cache if it fits.
 constexpr int kSumBlock = 256;
-constexpr uint64_t kSumChunk = 16384; // elements per work-group
+constexpr uint64_t kSumChunk = 65536; // elements per work-group
 
 __device__ __forceinline__ double blockSum(double v, double* lds) {
 #pragma unroll
@@ -266,10 +267,12 @@ __global__ __launch_bounds__(kSumBlock) void expSumKernel(const float* x, uint64
   double acc = 0.0;
   if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0 && end - begin == kSumChunk) {
     const v4f* x4 = reinterpret_cast<const v4f*>(x + begin);
-#pragma unroll 4
+#pragma unroll 8
     for (uint32_t i = threadIdx.x; i < kSumChunk / 4; i += kSumBlock) {
       const v4f v = x4[i];
-      acc += (double(expf(v.x)) + double(expf(v.y))) + (double(expf(v.z)) + double(expf(v.w)));
+      // four terms are added in fp32 (two roundings, 1.2e-7 relative at worst),
+      // everything above that in fp64
+      acc += double((expf(v.x) + expf(v.y)) + (expf(v.z) + expf(v.w)));
     }
   } else {
     for (uint64_t i = begin + threadIdx.x; i < end; i += kSumBlock) acc += double(expf(x[i]));
