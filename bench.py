@@ -334,6 +334,26 @@ def bench_graphs():
             "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
             "launches_per_evaluate": 4, "uploads_per_evaluate": int(c.copies_to_device // 55)}
         log(f"logreg forward through the plugin: {out['logreg_forward']['evaluate_us']} us per evaluation")
+    # the same forward pass with the extended (fused) builtins: 2 launches instead of 4
+    with harness.Harness(plugin=LIB_PLUGIN) as h:
+        X, W, B, Y = h.input(x), h.input(w), h.input(bias), h.input(y)
+        h.end_cluster()
+        p = h.fmatmul_fadd_fsigmoid(False, False, X, W, 1.0, B, 1.0)
+        h.end_cluster()
+        # flogloss consumes the sigmoid; the fused sigmoid+logloss would need the pre-activation,
+        # which the first fused launch does not keep
+        loss = h.flogloss(p, Y)
+        h.end_cluster()
+        for _ in range(5):
+            h.run()
+        ts = []
+        for _ in range(50):
+            t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
+        out["logreg_forward_fused"] = {
+            "workload": "same inputs; fmatmul_f_f_fadd_fsigmoid -> flogloss (extended builtins)",
+            "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
+            "launches_per_evaluate": 2}
+        log(f"logreg forward, fused builtins: {out['logreg_forward_fused']['evaluate_us']} us per evaluation")
     rng = np.random.default_rng(71)
     x = rng.random((1024, 1024), dtype=np.float32)
     w1 = (rng.standard_normal((1024, 4096)) / 32).astype(np.float32)

@@ -222,6 +222,30 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
                     uint64_t height, uint64_t width, uint64_t window0,
                     uint64_t window1, uint64_t stride0, uint64_t stride1);
 
+/* ---- Extended (fused) builtins -------------------------------------------------
+ * The reference's design allows runtimes to offer fused builtins that
+ * optimisation passes may emit, never the graph compiler itself
+ * (docs/design/llvm/04_builtins.md:12-19); it defines none.  These three fuse
+ * the chains its model graphs contain (matmul -> fadd -> fsigmoid, matmul ->
+ * fsigmoid, fsigmoid -> flogloss).  Each applies the operations of the
+ * builtins it replaces, in their order, so its result is bit-identical to
+ * running them one after the other. */
+/* out = fsigmoid(opA(A) * opB(B)) */
+int polar_hip_fmatmul_fsigmoid(polar_hip_device* dev, int transA, int transB,
+                               const float* a, const float* b, float* out,
+                               uint64_t m, uint64_t n, uint64_t k);
+/* out = fsigmoid(fadd(opA(A) * opB(B), scaleProduct, bias, scaleBias)); bias is
+ * M x N (fadd does not broadcast) */
+int polar_hip_fmatmul_fadd_fsigmoid(polar_hip_device* dev, int transA,
+                                    int transB, const float* a, const float* b,
+                                    float scaleProduct, const float* bias,
+                                    float scaleBias, float* out, uint64_t m,
+                                    uint64_t n, uint64_t k);
+/* out = flogloss(fsigmoid(in), groundTruth) */
+int polar_hip_fsigmoid_flogloss(polar_hip_device* dev, const float* in,
+                                const float* groundTruth, float* out,
+                                uint64_t n);
+
 #ifdef __cplusplus
 }
 #endif

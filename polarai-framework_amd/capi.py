@@ -92,6 +92,9 @@ SIGNATURES = {
     "polar_hip_fsoftmax": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fconv2d": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64]),
     "polar_hip_fpool": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64, _u64]),
+    "polar_hip_fmatmul_fsigmoid": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
+    "polar_hip_fmatmul_fadd_fsigmoid": (_i, [_vp, _i, _i, _vp, _vp, _f, _vp, _f, _vp, _u64, _u64, _u64]),
+    "polar_hip_fsigmoid_flogloss": (_i, [_vp, _vp, _vp, _vp, _u64]),
 }
 
 _lib = None
@@ -305,6 +308,19 @@ class Device:
     def fpool(self, x, out, height, width, window, stride):
         _check(self.lib, self.lib.polar_hip_fpool(self.handle, x.ptr, out.ptr, height, width,
                                                   window[0], window[1], stride[0], stride[1]))
+
+    def fmatmul_fsigmoid(self, trans_a, trans_b, a, b, out, m, n, k):
+        _check(self.lib, self.lib.polar_hip_fmatmul_fsigmoid(self.handle, int(trans_a), int(trans_b), a.ptr, b.ptr,
+                                                             out.ptr, m, n, k))
+
+    def fmatmul_fadd_fsigmoid(self, trans_a, trans_b, a, b, scale_product, bias, scale_bias, out, m, n, k):
+        _check(self.lib, self.lib.polar_hip_fmatmul_fadd_fsigmoid(self.handle, int(trans_a), int(trans_b), a.ptr,
+                                                                  b.ptr, scale_product, bias.ptr, scale_bias,
+                                                                  out.ptr, m, n, k))
+
+    def fsigmoid_flogloss(self, x, truth, out, n=None):
+        _check(self.lib, self.lib.polar_hip_fsigmoid_flogloss(self.handle, x.ptr, truth.ptr, out.ptr,
+                                                              out.count if n is None else n))
 
     def fmatmul(self, trans_a, trans_b, a, b, c, m, n, k):
         _check(self.lib, self.lib.polar_hip_fmatmul(

@@ -74,6 +74,14 @@ struct SigmoidOp { // sycl/kernels/Sigmoid.hpp:32-41
     return r;
   }
 };
+// Extended builtin: flogloss(fsigmoid(x), truth) in one pass, the operations of
+// the two functors above in the same order (bit-identical to the chain).
+struct SigmoidLogLossOp {
+  static constexpr int NIN = 2;
+  __device__ __forceinline__ float apply(float x, float g) const {
+    return LogLossOp{}.apply(SigmoidOp{}.apply(x, 0.0f), g);
+  }
+};
 struct ScaleOp { // sycl/kernels/MulConcat.hpp:33-35 (g = gradient[0])
   static constexpr int NIN = 1;
   float g;
@@ -386,6 +394,13 @@ int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out, uint6
   polar_hip_free(dev, workspace); // stream-ordered: reused only by later work
   if (e != hipSuccess) return failHip(e, "fsoftmax launch");
   return st;
+}
+
+int polar_hip_fsigmoid_flogloss(polar_hip_device* dev, const float* in,
+                                const float* groundTruth, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (in && groundTruth && out), "null tensor");
+  return launchEw<SigmoidLogLossOp>(dev, SigmoidLogLossOp{}, nullptr, in, groundTruth, out, n);
 }
 
 } // extern "C"

@@ -61,7 +61,35 @@ struct MatmulArgs {
   uint32_t tilesM, tilesN;
   uint32_t kSplits;   // work-groups [s*tiles, (s+1)*tiles) handle split s
   uint32_t kPerSplit; // multiple of BK
+  // fused epilogue of the extended builtins (kEpi*); applied where the final
+  // value of an element is produced: the kernel's store, or the split-K
+  // reduction
+  int epilogue;
+  const float* bias;  // M x N, dense (the framework's fadd does not broadcast)
+  float scaleAcc, scaleBias;
 };
+
+constexpr int kEpiNone = 0;
+constexpr int kEpiSigmoid = 1;     // sigmoid(acc)
+constexpr int kEpiAddSigmoid = 2;  // sigmoid(scaleAcc*acc + scaleBias*bias)
+
+// The same operations, in the same order, as the separate fadd and fsigmoid
+// kernels apply (sycl/kernels/AddNaive.hpp:33-35, Sigmoid.hpp:32-41), so the
+// fused result is bit-identical to the chain of builtins it replaces.
+__device__ __forceinline__ float applyEpilogue(int epilogue, float acc, const float* bias,
+                                               float scaleAcc, float scaleBias, size_t idx) {
+  if (epilogue == kEpiNone) return acc;
+  float x = acc;
+  if (epilogue == kEpiAddSigmoid) x = scaleAcc * acc + scaleBias * bias[idx];
+  const float eps = 1e-5f;
+  float r = 1.0f / (1.0f + expf(-x));
+  if (fabsf(r - 1.0f) < eps) {
+    r = 1.0f - eps;
+  } else if (fabsf(r) < eps) {
+    r = eps;
+  }
+  return r;
+}
 
 // Fetch of one operand tile (BX x BK) from HBM into registers, and its store
 // into the k-major LDS stage.  KCONTIG: element (x, k) lives at
@@ -261,8 +289,12 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
       for (int r = 0; r < 16; ++r) {
         const uint32_t row =
             m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
-        if (!EDGE || (row < p.M && col < p.N))
-          out[size_t(row) * p.N + col] = acc[i][j][r];
+        if (!EDGE || (row < p.M && col < p.N)) {
+          const size_t idx = size_t(row) * p.N + col;
+          out[idx] = p.kSplits > 1 ? acc[i][j][r]
+                                   : applyEpilogue(p.epilogue, acc[i][j][r], p.bias,
+                                                   p.scaleAcc, p.scaleBias, idx);
+        }
       }
     }
   }
@@ -271,12 +303,14 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
 // C[i] = partial[0][i] + partial[1][i] + ... in split order.
 __global__ __launch_bounds__(256) void splitKReduceKernel(const float* __restrict__ partial,
                                                           float* __restrict__ c,
-                                                          uint64_t count, uint32_t splits) {
+                                                          uint64_t count, uint32_t splits,
+                                                          int epilogue, const float* bias,
+                                                          float scaleAcc, float scaleBias) {
   const uint64_t stride = uint64_t(gridDim.x) * 256;
   for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) {
-    float acc = partial[i];
+    float acc = splits != 0 ? partial[i] : 0.0f; // no splits: an empty contraction
     for (uint32_t s = 1; s < splits; ++s) acc += partial[uint64_t(s) * count + i];
-    c[i] = acc;
+    c[i] = applyEpilogue(epilogue, acc, bias, scaleAcc, scaleBias, i);
   }
 }
 
@@ -333,7 +367,7 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
       if (grid > cap) grid = cap;
       hipError_t e = launchKernel(dev, splitKReduceKernel, dim3(static_cast<unsigned>(grid)),
                                   dim3(256), static_cast<const float*>(workspace), c, count,
-                                  splits);
+                                  splits, p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
       if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
     }
     // stream-ordered pool: the block may be handed out again only to work
@@ -399,9 +433,10 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
 
 } // namespace
 
-extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
-                                 const float* a, const float* b, float* c,
-                                 uint64_t m, uint64_t n, uint64_t k) {
+namespace {
+int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const float* a,
+                       const float* b, float* c, uint64_t m, uint64_t n, uint64_t k,
+                       int epilogue, const float* bias, float scaleAcc, float scaleBias) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   if (m == 0 || n == 0) return POLAR_HIP_OK;
   POLAR_HIP_REQUIRE(c != nullptr, "null output");
@@ -409,13 +444,21 @@ extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
   POLAR_HIP_REQUIRE(m < (1ull << 31) && n < (1ull << 31) && k < (1ull << 31),
                     "dimension does not fit 31 bits");
   POLAR_HIP_REQUIRE(c != a && c != b, "output aliases an operand");
+  POLAR_HIP_REQUIRE(epilogue != kEpiAddSigmoid || bias != nullptr, "null bias");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  MatmulArgs p{a, b, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+               static_cast<uint32_t>(k), 0, 0, 1, 0, epilogue, bias, scaleAcc, scaleBias};
   if (k == 0) {
     // Empty contraction: the reference's loop leaves acc = 0 and stores it.
-    return polar_hip_ffill(dev, 0.0f, c, m * n);
+    if (epilogue == kEpiNone) return polar_hip_ffill(dev, 0.0f, c, m * n);
+    uint64_t grid = (m * n + 255) / 256;
+    const uint64_t cap = uint64_t(dev->info.compute_units) * 16;
+    if (grid > cap) grid = cap;
+    POLAR_HIP_TRY(launchKernel(dev, splitKReduceKernel, dim3(static_cast<unsigned>(grid)),
+                               dim3(256), static_cast<const float*>(nullptr), c, m * n, 0u,
+                               epilogue, bias, scaleAcc, scaleBias));
+    return POLAR_HIP_OK;
   }
-  MatmulArgs p{a, b, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
-               static_cast<uint32_t>(k), 0, 0, 1, 0};
   const bool ta = transA != 0, tb = transB != 0;
   const MatmulPlan plan = planMatmul(p.M, p.N, p.K, dev->info.compute_units);
   switch (plan.config) {
@@ -426,4 +469,27 @@ extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
   case 4: return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p, plan.splits);
   default: return launchTile<32, 32, 32, 1, 1>(dev, ta, tb, p, plan.splits);
   }
+}
+} // namespace
+
+extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
+                                 const float* a, const float* b, float* c,
+                                 uint64_t m, uint64_t n, uint64_t k) {
+  return matmulWithEpilogue(dev, transA, transB, a, b, c, m, n, k, kEpiNone, nullptr, 1.0f, 1.0f);
+}
+
+extern "C" int polar_hip_fmatmul_fsigmoid(polar_hip_device* dev, int transA, int transB,
+                                          const float* a, const float* b, float* out,
+                                          uint64_t m, uint64_t n, uint64_t k) {
+  return matmulWithEpilogue(dev, transA, transB, a, b, out, m, n, k, kEpiSigmoid, nullptr, 1.0f,
+                            1.0f);
+}
+
+extern "C" int polar_hip_fmatmul_fadd_fsigmoid(polar_hip_device* dev, int transA, int transB,
+                                               const float* a, const float* b, float scaleProduct,
+                                               const float* bias, float scaleBias, float* out,
+                                               uint64_t m, uint64_t n, uint64_t k) {
+  POLAR_HIP_REQUIRE(bias != out, "output aliases the bias");
+  return matmulWithEpilogue(dev, transA, transB, a, b, out, m, n, k, kEpiAddSigmoid, bias,
+                            scaleProduct, scaleBias);
 }

@@ -237,6 +237,23 @@ class Harness:
         self.node("ftranspose", [a, out], 1)
         return out
 
+    # extended (fused) builtins
+    def fsigmoid_flogloss(self, x, truth, out=None):
+        return self._binary("fsigmoid_flogloss", x, truth, out)
+
+    def fmatmul_fsigmoid(self, ta, tb, a, b, out=None):
+        m = a.shape[1] if ta else a.shape[0]
+        n = b.shape[0] if tb else b.shape[1]
+        out = out or self.tensor(m, n)
+        self.node(f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'}_fsigmoid", [a, b, out], 2)
+        return out
+
+    def fmatmul_fadd_fsigmoid(self, ta, tb, a, b, scale_product, bias, scale_bias, out=None):
+        out = out or self.tensor(*bias.shape)
+        self.node(f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'}_fadd_fsigmoid",
+                  [a, b, float(scale_product), bias, float(scale_bias), out], 5)
+        return out
+
     def frelu(self, x, out=None):
         out = out or self.tensor(*x.shape)
         self.node("frelu", [x, out], 1)

@@ -96,6 +96,24 @@ uint64_t countArg(const LaunchCommand& cmd, uint64_t i) {
   return static_cast<uint64_t>(v);
 }
 
+void checkMatmulShapes(const LaunchCommand& cmd, bool ta, bool tb, const TensorArg& a,
+                       const TensorArg& b, const TensorArg& c, uint64_t* m, uint64_t* n,
+                       uint64_t* k) {
+  if (a.info->dims != 2 || b.info->dims != 2 || c.info->dims != 2)
+    fatal("%s: operands must be 2-D", cmd.nativeKernelName);
+  *m = c.info->shape[0];
+  *n = c.info->shape[1];
+  *k = ta ? a.info->shape[0] : a.info->shape[1];
+  const uint64_t am = ta ? a.info->shape[1] : a.info->shape[0];
+  const uint64_t bk = tb ? b.info->shape[1] : b.info->shape[0];
+  const uint64_t bn = tb ? b.info->shape[0] : b.info->shape[1];
+  if (am != *m || bk != *k || bn != *n)
+    fatal("%s: shapes do not agree: opA is %llux%llu, opB is %llux%llu, C is %llux%llu",
+          cmd.nativeKernelName, (unsigned long long)am, (unsigned long long)*k,
+          (unsigned long long)bk, (unsigned long long)bn, (unsigned long long)*m,
+          (unsigned long long)*n);
+}
+
 using Launcher = void (*)(HipDevice&, BackendAllocator&, LaunchCommand&);
 
 // [0]a T [1]scaleA D [2]b T [3]scaleB D [4]c T; range = c
@@ -221,20 +239,41 @@ void launchTranspose(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
 template <bool TA, bool TB>
 void launchMatMul(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
   TensorArg a = tensorArg(cmd, 0), b = tensorArg(cmd, 1), c = tensorArg(cmd, 2);
-  if (a.info->dims != 2 || b.info->dims != 2 || c.info->dims != 2)
-    fatal("%s: operands must be 2-D", cmd.nativeKernelName);
-  const uint64_t m = c.info->shape[0], n = c.info->shape[1];
-  const uint64_t k = TA ? a.info->shape[0] : a.info->shape[1];
-  const uint64_t am = TA ? a.info->shape[1] : a.info->shape[0];
-  const uint64_t bk = TB ? b.info->shape[1] : b.info->shape[0];
-  const uint64_t bn = TB ? b.info->shape[0] : b.info->shape[1];
-  if (am != m || bk != k || bn != n)
-    fatal("%s: shapes do not agree: opA is %llux%llu, opB is %llux%llu, C is %llux%llu",
-          cmd.nativeKernelName, (unsigned long long)am, (unsigned long long)k,
-          (unsigned long long)bk, (unsigned long long)bn, (unsigned long long)m,
-          (unsigned long long)n);
+  uint64_t m, n, k;
+  checkMatmulShapes(cmd, TA, TB, a, b, c, &m, &n, &k);
   checkStatus(polar_hip_fmatmul(d.native(), TA, TB, d.resolve(al, a.record),
                                 d.resolve(al, b.record), d.resolve(al, c.record), m, n, k),
+              cmd.nativeKernelName);
+}
+
+// Extended (fused) builtins; none of them is emitted by the graph compiler
+// (docs/design/llvm/04_builtins.md:12-19), an optimisation pass would.
+// fmatmul_X_Y_fsigmoid: [0]A T [1]B T [2]out T
+template <bool TA, bool TB>
+void launchMatMulSigmoid(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
+  TensorArg a = tensorArg(cmd, 0), b = tensorArg(cmd, 1), c = tensorArg(cmd, 2);
+  uint64_t m, n, k;
+  checkMatmulShapes(cmd, TA, TB, a, b, c, &m, &n, &k);
+  checkStatus(polar_hip_fmatmul_fsigmoid(d.native(), TA, TB, d.resolve(al, a.record),
+                                         d.resolve(al, b.record), d.resolve(al, c.record), m,
+                                         n, k),
+              cmd.nativeKernelName);
+}
+
+// fmatmul_X_Y_fadd_fsigmoid: [0]A T [1]B T [2]scaleProduct D [3]bias T [4]scaleBias D [5]out T
+// (the matmul's operands followed by fadd's remaining ones)
+template <bool TA, bool TB>
+void launchMatMulAddSigmoid(HipDevice& d, BackendAllocator& al, LaunchCommand& cmd) {
+  TensorArg a = tensorArg(cmd, 0), b = tensorArg(cmd, 1), bias = tensorArg(cmd, 3),
+            c = tensorArg(cmd, 5);
+  const float sp = scalarArg(cmd, 2), sb = scalarArg(cmd, 4);
+  uint64_t m, n, k;
+  checkMatmulShapes(cmd, TA, TB, a, b, c, &m, &n, &k);
+  needAtLeast(cmd, bias, c.count);
+  checkStatus(polar_hip_fmatmul_fadd_fsigmoid(d.native(), TA, TB, d.resolve(al, a.record),
+                                              d.resolve(al, b.record), sp,
+                                              d.resolve(al, bias.record), sb,
+                                              d.resolve(al, c.record), m, n, k),
               cmd.nativeKernelName);
 }
 
@@ -263,6 +302,15 @@ const TableEntry kTable[] = {
     {"fmatmul_f_t", launchMatMul<false, true>},
     {"fmatmul_t_f", launchMatMul<true, false>},
     {"fmatmul_t_t", launchMatMul<true, true>},
+    {"fsigmoid_flogloss", launchBinary<polar_hip_fsigmoid_flogloss, false>},
+    {"fmatmul_f_f_fsigmoid", launchMatMulSigmoid<false, false>},
+    {"fmatmul_f_t_fsigmoid", launchMatMulSigmoid<false, true>},
+    {"fmatmul_t_f_fsigmoid", launchMatMulSigmoid<true, false>},
+    {"fmatmul_t_t_fsigmoid", launchMatMulSigmoid<true, true>},
+    {"fmatmul_f_f_fadd_fsigmoid", launchMatMulAddSigmoid<false, false>},
+    {"fmatmul_f_t_fadd_fsigmoid", launchMatMulAddSigmoid<false, true>},
+    {"fmatmul_t_f_fadd_fsigmoid", launchMatMulAddSigmoid<true, false>},
+    {"fmatmul_t_t_fadd_fsigmoid", launchMatMulAddSigmoid<true, true>},
 };
 
 } // namespace

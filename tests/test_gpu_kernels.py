@@ -385,3 +385,67 @@ def test_pool_bit_exact(dev, shape, window, stride):
         assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
         assert np.all(got[ref.size:] == -7.0)
         dx.free(); dout.free()
+
+
+# ---- extended (fused) builtins ----------------------------------------------------
+
+FUSED_SHAPES = [(256, 10, 784), (64, 64, 64), (33, 127, 4096), (300, 257, 129), (1024, 1024, 512), (5, 3, 0)]
+
+
+@pytest.mark.parametrize("mnk", FUSED_SHAPES)
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_fused_matmul_epilogues_equal_the_unfused_chain(dev, ta, tb, mnk):
+    """fmatmul_fsigmoid / fmatmul_fadd_fsigmoid against running fmatmul, fadd and
+    fsigmoid one after the other on the device (must be identical bit for bit, for
+    plain and for split-K plans), and against the oracle's chain within the
+    matmul tolerance."""
+    m, n, k = mnk
+    _say("fused matmul", ta, tb, mnk)
+    rng = np.random.default_rng(1100 + m + k)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, max(k, 1))
+    a, b = parity.normal(rng, sa, 0.3), parity.normal(rng, sb, 0.3)
+    bias = parity.normal(rng, (m, n))
+    da, db, dbias = dev.array(a), dev.array(b), dev.array(bias)
+    prod, summed, chain, fused = dev.empty(m * n), dev.empty(m * n), dev.empty(m * n), dev.empty(m * n)
+    dev.fmatmul(ta, tb, da, db, prod, m, n, k)
+    # sigmoid(product)
+    dev.fsigmoid(prod, chain)
+    dev.fmatmul_fsigmoid(ta, tb, da, db, fused, m, n, k)
+    assert np.array_equal(fused.download(), chain.download())
+    # sigmoid(0.75 * product - 0.5 * bias)
+    dev.fadd(prod, 0.75, dbias, -0.5, summed)
+    dev.fsigmoid(summed, chain)
+    dev.fmatmul_fadd_fsigmoid(ta, tb, da, db, 0.75, dbias, -0.5, fused, m, n, k)
+    got = fused.download()
+    assert np.array_equal(got, chain.download())
+    if k > 0:
+        ref = o.fsigmoid(o.fadd(o.fmatmul(ta, tb, a, b), 0.75, bias, -0.5))
+        assert parity.frobenius_rel_error(got.reshape(m, n), ref) <= parity.MATMUL_FRO_REL
+    else:
+        assert np.array_equal(got.reshape(m, n), o.fsigmoid(o.fadd(np.zeros((m, n), np.float32), 0.75, bias, -0.5)))
+    for t in (da, db, dbias, prod, summed, chain, fused):
+        t.free()
+
+
+@pytest.mark.parametrize("n", [1, 5, 1000, 65536 + 7, 1000003])
+def test_fused_sigmoid_logloss_equals_the_unfused_chain(dev, n):
+    _say("fused sigmoid+logloss n=", n)
+    rng = np.random.default_rng(1200 + n)
+    x = parity.normal(rng, n, 3.0)
+    y = (rng.random(n) < 0.3).astype(np.float32)
+    dx, dy, dp, chain, fused = dev.array(x), dev.array(y), dev.empty(n), dev.empty(n), dev.empty(n)
+    dev.fsigmoid(dx, dp)
+    dev.flogloss(dp, dy, chain)
+    dev.fsigmoid_flogloss(dx, dy, fused)
+    got = fused.download()
+    assert np.array_equal(got, chain.download())
+    # per kernel against the oracle, as for the unfused builtins: the sigmoid the
+    # device produced, then the oracle's logloss of exactly those values (a chain of
+    # two tolerances is not a tolerance: log(1 - p + eps) amplifies the last bit of p
+    # where p saturates)
+    p = dp.download()
+    assert parity.elementwise_rel_error(p, o.fsigmoid(x)) <= parity.ELEMENTWISE_REL
+    assert parity.elementwise_rel_error(got, o.flogloss(p, y)) <= parity.ELEMENTWISE_REL
+    for t in (dx, dy, dp, chain, fused):
+        t.free()

@@ -324,3 +324,29 @@ def test_native_kernel_wins_over_a_program_kernel_of_the_same_node(h):
     h.end_cluster()
     h.run()
     assert np.array_equal(h.read(out), np.arange(8, dtype=np.float32) * 5)
+
+
+def test_fused_builtins_through_plugin(h):
+    """The logistic-regression forward pass as two fused launches equals the four-kernel graph."""
+    rng = np.random.default_rng(54)
+    x = rng.random((256, 784), dtype=np.float32)
+    w = parity.normal(rng, (784, 10), 0.01)
+    bias = parity.normal(rng, (256, 10), 0.1)
+    y = (rng.random((256, 10)) < 0.1).astype(np.float32)
+    X, W, B, Y = h.input(x), h.input(w), h.input(bias), h.input(y)
+    h.end_cluster()
+    z = h.fmatmul(False, False, X, W)
+    fused_p = h.fmatmul_fadd_fsigmoid(False, False, X, W, 1.0, B, 1.0)
+    h.end_cluster()
+    s = h.fadd(z, 1.0, B, 1.0)
+    h.end_cluster()
+    p = h.fsigmoid(s)
+    fused_loss = h.fsigmoid_flogloss(s, Y)
+    h.end_cluster()
+    loss = h.flogloss(p, Y)
+    h.end_cluster()
+    h.run()
+    assert np.array_equal(h.read(fused_p), h.read(p))
+    assert np.array_equal(h.read(fused_loss), h.read(loss))
+    ref = o.fsigmoid(o.fadd(o.fmatmul(False, False, x, w), 1.0, bias, 1.0))
+    assert parity.elementwise_rel_error(h.read(p), ref) <= parity.ELEMENTWISE_REL
