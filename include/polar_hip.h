@@ -92,7 +92,11 @@ int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out);
  * Stand in for Device::copyToDevice / copyToHost of the reference's runtimes
  * (src/backend/generic/runtime/cuda/CudaDevice.hpp:52-61,
  *  src/backend/generic/runtime/sycl/SYCLDevice.h:81-112): ordered after all
- * work already enqueued on the device, complete when the call returns. */
+ * work already enqueued on the device.  copy_to_host is complete when the call
+ * returns.  copy_to_device has consumed src_host when it returns (the caller
+ * may reuse it at once); for transfers of up to 4 MiB the DMA into dst_device
+ * may still be in flight on the device's stream, where every later kernel,
+ * copy and event of this library is ordered behind it. */
 int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
                              const void* src_host, uint64_t bytes);
 int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,

@@ -35,9 +35,13 @@ struct polar_hip_device {
   std::vector<polar_hip_event*> idleEvents;
   std::vector<polar_hip_event*> allEvents;
 
-  // pinned bounce buffer for small and medium host<->device copies
+  // ring of pinned slots for small and medium host<->device copies; a slot
+  // is busy until the event recorded behind its transfer has completed
   std::mutex stagingMu;
   void* staging = nullptr;
+  hipEvent_t slotEvent[8] = {};
+  bool slotBusy[8] = {};
+  int nextSlot = 0;
 
   // armed by polar_hip_time_next_kernel: the next kernel launch carries these
   // as its start/stop events

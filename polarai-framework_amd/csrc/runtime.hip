@@ -109,7 +109,10 @@ int polar_hip_device_close(polar_hip_device* dev) {
     (void)hipEventDestroy(e->ev);
     delete e;
   }
-  if (dev->staging) (void)hipHostFree(dev->staging);
+  if (dev->staging) {
+    for (hipEvent_t e : dev->slotEvent) (void)hipEventDestroy(e);
+    (void)hipHostFree(dev->staging);
+  }
   (void)hipStreamDestroy(dev->stream);
   delete dev;
   return POLAR_HIP_OK;
@@ -211,21 +214,57 @@ int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out) {
 // Host memory handed in by the framework is pageable.  The driver's pageable
 // path is fast for large transfers (30 GB/s up, 18 GB/s down, measured) but has
 // a high fixed cost for small and medium ones (110 us for 256 KiB), which is
-// what graph inputs and read-backs mostly are.  Those go through a pinned
-// bounce buffer instead: one host memcpy plus one DMA.
+// what graph inputs and read-backs mostly are.  Transfers of up to 4 MiB go
+// through a ring of pinned 512 KiB slots instead:
+//  * upload: the source is copied into a slot and the DMA is enqueued on the
+//    device's stream; the call returns without waiting for it (the caller's
+//    buffer is already free, and everything that uses the destination is
+//    ordered after the DMA on the same stream).  A slot is reused only after
+//    the event recorded behind its DMA has completed.
+//  * download: the DMAs of all chunks are enqueued first, then each chunk is
+//    copied out as soon as its event completes, so the host copy of one chunk
+//    overlaps the DMA of the next.
 namespace {
-constexpr uint64_t kStagingBytes = 4ull << 20;
+constexpr uint64_t kSlotBytes = 512ull << 10;
+constexpr int kSlots = 8;
+constexpr uint64_t kStagingBytes = kSlotBytes * kSlots;
 
-void* stagingBuffer(polar_hip_device* dev) {
-  if (dev->staging == nullptr) {
-    void* p = nullptr;
-    if (hipHostMalloc(&p, kStagingBytes, hipHostMallocDefault) != hipSuccess) {
-      (void)hipGetLastError();
-      return nullptr;
-    }
-    dev->staging = p;
+// called with dev->stagingMu held
+bool stagingReady(polar_hip_device* dev) {
+  if (dev->staging != nullptr) return true;
+  void* p = nullptr;
+  if (hipHostMalloc(&p, kStagingBytes, hipHostMallocDefault) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
   }
-  return dev->staging;
+  for (int i = 0; i < kSlots; ++i) {
+    if (hipEventCreateWithFlags(&dev->slotEvent[i], hipEventDisableTiming) != hipSuccess) {
+      (void)hipGetLastError();
+      for (int k = 0; k < i; ++k) (void)hipEventDestroy(dev->slotEvent[k]);
+      (void)hipHostFree(p);
+      return false;
+    }
+    dev->slotBusy[i] = false;
+  }
+  dev->staging = p;
+  return true;
+}
+
+// next slot of the ring, idle (its previous transfer has completed)
+hipError_t acquireSlot(polar_hip_device* dev, int* slot) {
+  const int s = dev->nextSlot;
+  dev->nextSlot = (s + 1) % kSlots;
+  if (dev->slotBusy[s]) {
+    hipError_t e = hipEventSynchronize(dev->slotEvent[s]);
+    if (e != hipSuccess) return e;
+    dev->slotBusy[s] = false;
+  }
+  *slot = s;
+  return hipSuccess;
+}
+
+char* slotMemory(polar_hip_device* dev, int slot) {
+  return static_cast<char*>(dev->staging) + uint64_t(slot) * kSlotBytes;
 }
 } // namespace
 
@@ -238,11 +277,17 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   if (bytes <= kStagingBytes) {
     std::lock_guard<std::mutex> g(dev->stagingMu);
-    if (void* pinned = stagingBuffer(dev)) {
-      memcpy(pinned, src_host, bytes);
-      POLAR_HIP_TRY(hipMemcpyAsync(dst_device, pinned, bytes, hipMemcpyHostToDevice,
-                                   dev->stream));
-      POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+    if (stagingReady(dev)) {
+      for (uint64_t off = 0; off < bytes; off += kSlotBytes) {
+        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
+        int slot;
+        POLAR_HIP_TRY(acquireSlot(dev, &slot));
+        memcpy(slotMemory(dev, slot), static_cast<const char*>(src_host) + off, n);
+        POLAR_HIP_TRY(hipMemcpyAsync(static_cast<char*>(dst_device) + off, slotMemory(dev, slot),
+                                     n, hipMemcpyHostToDevice, dev->stream));
+        POLAR_HIP_TRY(hipEventRecord(dev->slotEvent[slot], dev->stream));
+        dev->slotBusy[slot] = true;
+      }
       return POLAR_HIP_OK;
     }
   }
@@ -261,11 +306,25 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   if (bytes <= kStagingBytes) {
     std::lock_guard<std::mutex> g(dev->stagingMu);
-    if (void* pinned = stagingBuffer(dev)) {
-      POLAR_HIP_TRY(hipMemcpyAsync(pinned, src_device, bytes, hipMemcpyDeviceToHost,
-                                   dev->stream));
-      POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
-      memcpy(dst_host, pinned, bytes);
+    if (stagingReady(dev)) {
+      int slots[kSlots];
+      int chunks = 0;
+      for (uint64_t off = 0; off < bytes; off += kSlotBytes, ++chunks) {
+        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
+        POLAR_HIP_TRY(acquireSlot(dev, &slots[chunks]));
+        POLAR_HIP_TRY(hipMemcpyAsync(slotMemory(dev, slots[chunks]),
+                                     static_cast<const char*>(src_device) + off, n,
+                                     hipMemcpyDeviceToHost, dev->stream));
+        POLAR_HIP_TRY(hipEventRecord(dev->slotEvent[slots[chunks]], dev->stream));
+        dev->slotBusy[slots[chunks]] = true;
+      }
+      for (int c = 0; c < chunks; ++c) {
+        const uint64_t off = uint64_t(c) * kSlotBytes;
+        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
+        POLAR_HIP_TRY(hipEventSynchronize(dev->slotEvent[slots[c]]));
+        dev->slotBusy[slots[c]] = false;
+        memcpy(static_cast<char*>(dst_host) + off, slotMemory(dev, slots[c]), n);
+      }
       return POLAR_HIP_OK;
     }
   }
