@@ -90,6 +90,19 @@ inline hipError_t launchKernel(polar_hip_device* dev, void (*kernel)(KArgs...),
   return launchKernelLds(dev, kernel, grid, block, 0u, args...);
 }
 
+// Streaming stores for output that the kernel does not read again: the
+// non-temporal hint plus device-scope write-through (sc1), so the lines leave
+// the XCD's L2 as they are written instead of lingering there dirty.  Measured
+// on a 2^26-element copy: 84.0 us with the non-temporal hint alone, 81.5 us
+// with both (stores without any hint 88 us).
+typedef float polar_v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void streamStore(polar_v4f value, polar_v4f* address) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(address), "v"(value) : "memory");
+}
+__device__ __forceinline__ void streamStore(float value, float* address) {
+  asm volatile("global_store_dword %0, %1, off sc1 nt" : : "v"(address), "v"(value) : "memory");
+}
+
 inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
 }

@@ -153,7 +153,7 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
       }
     float* dst = p.out + uint64_t(y) * p.OW + x;
     if (x >= 0 && x + 3 < int64_t(p.OW)) {
-      __builtin_nontemporal_store(v4f{acc[0], acc[1], acc[2], acc[3]},
+      streamStore(v4f{acc[0], acc[1], acc[2], acc[3]},
                                   reinterpret_cast<v4f*>(dst));
     } else {
 #pragma unroll
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(kSegment) void conv2dDirectKernel(ConvArgs p) {
     const float* src = p.in + uint64_t(y + a) * p.W + uint64_t(x);
     for (uint32_t b = 0; b < p.KW; ++b) acc = src[b] * p.weights[a * p.KW + b] + acc;
   }
-  __builtin_nontemporal_store(acc, &p.out[uint64_t(y) * p.OW + uint64_t(x)]);
+  streamStore(acc, &p.out[uint64_t(y) * p.OW + uint64_t(x)]);
 }
 
 struct PoolArgs {
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kSegment) void poolKernel(PoolArgs p) {
           best = v > best ? v : best;
         }
       }
-      __builtin_nontemporal_store(best, &p.out[uint64_t(y) * p.OW + uint64_t(x)]);
+      streamStore(best, &p.out[uint64_t(y) * p.OW + uint64_t(x)]);
     }
   }
 }
