@@ -178,6 +178,7 @@ def main():
         result["transpose"] = bench_transpose(dev, args)
         result["matmul"] = bench_matmul(dev, args)
         result["next_builtins"] = bench_next_builtins(dev, da, n, args)
+        result["ragged"] = bench_ragged(dev, args)
     da.free(); db.free()
     dev.close()
     dev = None
@@ -267,6 +268,49 @@ def bench_next_builtins(dev, dx, n, args):
     assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
     for t in (dimg, dk, dpool):
         t.free()
+    return out
+
+
+def bench_ragged(dev, args):
+    """The ragged configuration: fadd/fmul on 1 000 003 elements and the two matmul
+    shapes 65536x127x33 / 33x65536x127 under both readings of the triple, (M, K, N)
+    and (M, N, K).  These are small: both roofline bounds are reported."""
+    out = {}
+    n = 1000003
+    rng = np.random.default_rng(9)
+    a, b = dev.array(rng.random(n, dtype=np.float32)), dev.array(rng.random(n, dtype=np.float32))
+    c = dev.empty(n)
+    for name, fn in (("fadd", lambda: dev.fadd(a, 1.0, b, 1.0, c)), ("fmul", lambda: dev.fmul(a, b, c))):
+        ms = time_kernel(dev, fn, args.warmup, args.steps)
+        gbs = 12 * n / (np.mean(ms) * 1e-3) / 1e9
+        out[f"{name}_{n}"] = {"us": round(float(np.mean(ms)) * 1e3, 2), "GB/s": round(gbs, 1),
+                              "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        log(f"{name} n={n}: {np.mean(ms) * 1e3:7.1f} us  {gbs:7.1f} GB/s")
+    for t in (a, b, c):
+        t.free()
+    for label, (m, nn, k) in (("65536x127x33 as (M,K,N)", (65536, 33, 127)), ("65536x127x33 as (M,N,K)", (65536, 127, 33)),
+                              ("33x65536x127 as (M,K,N)", (33, 127, 65536)), ("33x65536x127 as (M,N,K)", (33, 65536, 127))):
+        da = dev.array(rng.standard_normal((m, k), dtype=np.float32))
+        db = dev.array(rng.standard_normal((k, nn), dtype=np.float32))
+        dc = dev.empty(m * nn)
+        # split-K plans run two kernels: time the whole call with events around it
+        for _ in range(max(1, args.warmup)):
+            dev.fmatmul(0, 0, da, db, dc, m, nn, k)
+        dev.synchronize()
+        ms = []
+        for _ in range(max(5, args.steps)):
+            e0 = dev.record(); dev.fmatmul(0, 0, da, db, dc, m, nn, k); e1 = dev.record()
+            e1.synchronize(); ms.append(e0.elapsed_ms(e1)); e0.release(); e1.release()
+        t = float(np.mean(ms)) * 1e-3
+        flops, nbytes = 2.0 * m * nn * k, 4.0 * (m * k + k * nn + m * nn)
+        out[f"fmatmul_f_f {label}"] = {"M": m, "N": nn, "K": k, "us": round(t * 1e6, 2),
+                                       "GFLOP/s": round(flops / t / 1e9, 1),
+                                       "frac_mfma_fp32_peak": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+                                       "min_bytes_GB/s": round(nbytes / t / 1e9, 1),
+                                       "frac_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)}
+        log(f"fmatmul {label}: {t * 1e6:7.1f} us  {flops / t / 1e12:6.2f} TFLOP/s  {nbytes / t / 1e9:7.1f} GB/s of compulsory traffic")
+        for x in (da, db, dc):
+            x.free()
     return out
 
 
