@@ -72,6 +72,8 @@ def main():
                     help="elements per tensor in the sweep (default 2^26)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-matmul", action="store_true", help="skip the matmul/transpose legs")
+    ap.add_argument("--no-ragged", action="store_true",
+                    help="skip the ragged-shape leg (keeps a profile to one problem size per kernel)")
     ap.add_argument("--no-graphs", action="store_true",
                     help="skip the model-graph legs (keeps a profile to one problem size per kernel)")
     args = ap.parse_args()
@@ -178,7 +180,8 @@ def main():
         result["transpose"] = bench_transpose(dev, args)
         result["matmul"] = bench_matmul(dev, args)
         result["next_builtins"] = bench_next_builtins(dev, da, n, args)
-        result["ragged"] = bench_ragged(dev, args)
+        if not args.no_ragged:
+            result["ragged"] = bench_ragged(dev, args)
     da.free(); db.free()
     dev.close()
     dev = None

@@ -300,18 +300,57 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
   }
 }
 
-// C[i] = partial[0][i] + partial[1][i] + ... in split order.
-__global__ __launch_bounds__(256) void splitKReduceKernel(const float* __restrict__ partial,
-                                                          float* __restrict__ c,
-                                                          uint64_t count, uint32_t splits,
-                                                          int epilogue, const float* bias,
-                                                          float scaleAcc, float scaleBias) {
-  const uint64_t stride = uint64_t(gridDim.x) * 256;
-  for (uint64_t i = uint64_t(blockIdx.x) * 256 + threadIdx.x; i < count; i += stride) {
-    float acc = splits != 0 ? partial[i] : 0.0f; // no splits: an empty contraction
-    for (uint32_t s = 1; s < splits; ++s) acc += partial[uint64_t(s) * count + i];
-    c[i] = applyEpilogue(epilogue, acc, bias, scaleAcc, scaleBias, i);
+// C[i] = sum over splits of partial[s][i], in a fixed order: a work-group owns
+// 64 consecutive elements (one per lane); wave w adds the splits s = w, w+W,
+// w+2W, ... one after the other (loads four ahead), and the W wave sums are
+// then added in wave order.  Which lane adds what depends only on the indices,
+// so the result is the same on every run.  Many splits of a small C (33 x 127
+// in 256 splits) would otherwise be one long chain of dependent loads per
+// element (61 us for that shape; 6 us like this).
+// kReduceWaves = W is chosen from the number of splits (2, 4, 8 or 16).
+template <int kReduceWaves>
+__global__ __launch_bounds__(64 * kReduceWaves) void splitKReduceKernel(
+    const float* __restrict__ partial, float* __restrict__ c, uint64_t count, uint32_t splits,
+    int epilogue, const float* bias, float scaleAcc, float scaleBias) {
+  __shared__ float sums[kReduceWaves][64];
+  const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const uint64_t i = uint64_t(blockIdx.x) * 64 + lane;
+  float acc = 0.0f;
+  if (i < count) {
+    uint32_t s = wave;
+    for (; s + 3 * kReduceWaves < splits; s += 4 * kReduceWaves) {
+      const float v0 = partial[uint64_t(s) * count + i];
+      const float v1 = partial[uint64_t(s + kReduceWaves) * count + i];
+      const float v2 = partial[uint64_t(s + 2 * kReduceWaves) * count + i];
+      const float v3 = partial[uint64_t(s + 3 * kReduceWaves) * count + i];
+      acc = (((acc + v0) + v1) + v2) + v3;
+    }
+    for (; s < splits; s += kReduceWaves) acc += partial[uint64_t(s) * count + i];
   }
+  sums[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0 && i < count) {
+    float total = sums[0][lane];
+#pragma unroll
+    for (int w = 1; w < kReduceWaves; ++w) total += sums[w][lane];
+    c[i] = applyEpilogue(epilogue, total, bias, scaleAcc, scaleBias, i);
+  }
+}
+
+hipError_t launchReduce(polar_hip_device* dev, const float* partial, float* c, uint64_t count,
+                        uint32_t splits, const MatmulArgs& p) {
+  const dim3 grid(static_cast<unsigned>((count + 63) / 64));
+  if (splits <= 2)
+    return launchKernel(dev, splitKReduceKernel<2>, grid, dim3(128), partial, c, count, splits,
+                        p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
+  if (splits <= 4)
+    return launchKernel(dev, splitKReduceKernel<4>, grid, dim3(256), partial, c, count, splits,
+                        p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
+  if (splits <= 8)
+    return launchKernel(dev, splitKReduceKernel<8>, grid, dim3(512), partial, c, count, splits,
+                        p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
+  return launchKernel(dev, splitKReduceKernel<16>, grid, dim3(1024), partial, c, count, splits,
+                      p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
 }
 
 template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
@@ -362,12 +401,7 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
   else st = launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
   if (splits > 1) {
     if (st == POLAR_HIP_OK) {
-      uint64_t grid = (count + 255) / 256;
-      const uint64_t cap = uint64_t(dev->info.compute_units) * 16;
-      if (grid > cap) grid = cap;
-      hipError_t e = launchKernel(dev, splitKReduceKernel, dim3(static_cast<unsigned>(grid)),
-                                  dim3(256), static_cast<const float*>(workspace), c, count,
-                                  splits, p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
+      hipError_t e = launchReduce(dev, static_cast<const float*>(workspace), c, count, splits, p);
       if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
     }
     // stream-ordered pool: the block may be handed out again only to work
@@ -451,12 +485,9 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   if (k == 0) {
     // Empty contraction: the reference's loop leaves acc = 0 and stores it.
     if (epilogue == kEpiNone) return polar_hip_ffill(dev, 0.0f, c, m * n);
-    uint64_t grid = (m * n + 255) / 256;
-    const uint64_t cap = uint64_t(dev->info.compute_units) * 16;
-    if (grid > cap) grid = cap;
-    POLAR_HIP_TRY(launchKernel(dev, splitKReduceKernel, dim3(static_cast<unsigned>(grid)),
-                               dim3(256), static_cast<const float*>(nullptr), c, m * n, 0u,
-                               epilogue, bias, scaleAcc, scaleBias));
+    const uint64_t grid = (m * n + 63) / 64;
+    POLAR_HIP_REQUIRE(grid < (1ull << 31), "matrix too large for one launch");
+    POLAR_HIP_TRY(launchReduce(dev, nullptr, c, m * n, 0u, p));
     return POLAR_HIP_OK;
   }
   const bool ta = transA != 0, tb = transB != 0;
