@@ -43,9 +43,9 @@ SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
 # (profiles/bench_kernels_pmc_traffic.md).  They cannot be measured from inside
 # this process, so they are constants of the committed kernels.
 MEASURED_TRAFFIC_BYTES = {
-    "fadd": 804971090, "fmul": 804957950, "fdivide": 804973820, "fsigmoid": 536570873,
-    "fcopy": 536870912, "ffill": 268298771, "ftranspose": 703413924, "fmatmul": 469719808,
-    "frelu": 536692356, "fsoftmax": 805229623, "fconv2d": 537078775, "fpool": 335466015,
+    "fadd": 805290114, "fmul": 805280771, "fdivide": 805292759, "fsigmoid": 536890622,
+    "fcopy": 536870912, "ffill": 268459816, "ftranspose": 703813199, "fmatmul": 470152600,
+    "frelu": 536863659, "fsoftmax": 805432513, "fconv2d": 537560171, "fpool": 335545472,
 }
 T_ROWS, T_COLS = 12345, 6789
 MM = 4096
