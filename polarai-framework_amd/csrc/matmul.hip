@@ -238,10 +238,12 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const uint32_t nk = kEnd > kBegin ? (kEnd - kBegin + BK - 1) / BK : 0;
-  fa.load(p.A, lda, m0, kBegin, p.M, kEnd, t);
-  fb.load(p.B, ldb, n0, kBegin, p.N, kEnd, t);
-  fa.store(As[0], t);
-  fb.store(Bs[0], t);
+  if (nk != 0) { // uniform; the host never creates an empty split
+    fa.load(p.A, lda, m0, kBegin, p.M, kEnd, t);
+    fb.load(p.B, ldb, n0, kBegin, p.N, kEnd, t);
+    fa.store(As[0], t);
+    fb.store(Bs[0], t);
+  }
   __syncthreads();
 
   const int aBase = wm * WTM + (lane % 32);
@@ -376,8 +378,13 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
   p.tilesM = (p.M + BM - 1) / BM;
   p.tilesN = (p.N + BN - 1) / BN;
   const uint32_t kSteps = (p.K + BK - 1) / BK;
+  // Equal shares of whole k-steps; the number of splits is then what those
+  // shares need, so that no split starts at or beyond K (an empty split would
+  // prefetch its first tile from outside the operands).
+  const uint32_t stepsPerSplit = (kSteps + splits - 1) / splits;
+  splits = (kSteps + stepsPerSplit - 1) / stepsPerSplit;
   p.kSplits = splits;
-  p.kPerSplit = (kSteps + splits - 1) / splits * BK;
+  p.kPerSplit = stepsPerSplit * BK;
   // 16-byte fetches need aligned bases and a contiguous dimension that is a
   // multiple of 4 for both operands.
   const uint32_t contigA = ta ? p.M : p.K;

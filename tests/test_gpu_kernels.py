@@ -239,6 +239,23 @@ def test_matmul_long_k_is_split_and_reduced_in_order(dev, ta, tb, mnk):
         o.set_threads(1)
 
 
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+def test_matmul_split_count_never_leaves_an_empty_split(dev, ta, tb):
+    """256 x 256 x 16384: the planner asks for 96 splits of 1024 k-steps, i.e. 11
+    steps each, which only 94 splits can fill.  The operands are 16 MiB each,
+    exactly what the pool hands out, so a split starting beyond K would read
+    outside them."""
+    m, n, k = 256, 256, 16384
+    _say("split-k matmul without empty splits", ta, tb)
+    rng = np.random.default_rng(77 + 2 * ta + tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+    got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+    ref = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    assert parity.frobenius_rel_error(got, ref) <= 1e-5
+
+
 def test_matmul_overwrites_output(dev):
     # no beta: C is overwritten, stale contents must not leak
     rng = np.random.default_rng(31)
