@@ -42,6 +42,8 @@
 // come from a small cost model (planMatmul) of rounds x k-steps x step time.
 #include "internal.h"
 
+#include <cmath>
+
 
 using namespace polar_hip_detail;
 
@@ -457,9 +459,9 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
       double resident = groups / computeUnits;
       if (resident < 1) resident = 1;
       if (resident > t.residentGroups) resident = t.residentGroups;
-      const double rounds = groups <= double(computeUnits) * resident
-                                ? 1.0
-                                : groups / (double(computeUnits) * resident);
+      // whole rounds: the groups of a partly filled last round take as long as
+      // those of a full one (4097^3 on 256x256 tiles is 289 groups = 2 rounds)
+      const double rounds = std::ceil(groups / (double(computeUnits) * resident) - 1e-9);
       const double stepUs = resident * mfmaUs > 1.3 ? resident * mfmaUs : 1.3;
       double us = rounds * ((kSteps + s - 1) / s) * stepUs + 3.0;
       if (s > 1) us += 4.0 + double(m) * n * 4.0 * (s + 1) / 3.0e6;
