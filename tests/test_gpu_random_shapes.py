@@ -1,0 +1,95 @@
+"""Seeded random shapes for the kernels with index arithmetic (matmul in its four
+layouts, transpose, conv2d, pool): small enough for the oracle, awkward enough to
+hit every edge path (sizes around the tile sizes, odd pitches, bases off a line).
+Same bars as the fixed-shape tests: bit-exact for transpose/conv2d/pool, 1e-4
+relative Frobenius for matmul."""
+import numpy as np
+import pytest
+
+import parity
+import polar_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print(*a, flush=True)
+
+
+def _dims(rng, count, hi):
+    """sizes biased towards tile boundaries"""
+    special = np.array([1, 2, 3, 4, 5, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257])
+    special = special[special <= hi]
+    out = []
+    for _ in range(count):
+        out.append(int(rng.choice(special)) if rng.random() < 0.5 else int(rng.integers(1, hi + 1)))
+    return out
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_matmul(dev, seed):
+    rng = np.random.default_rng(5000 + seed)
+    m, n = _dims(rng, 2, 300)
+    k = _dims(rng, 1, 2500 if seed % 4 == 0 else 300)[0]
+    ta, tb = bool(rng.integers(2)), bool(rng.integers(2))
+    mis = int(rng.choice([0, 0, 1, 3]))
+    _say("random matmul", seed, (m, n, k), ta, tb, "misalign", mis)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+    da, db, dc = dev.array(a, mis), dev.array(b, mis), dev.empty(m * n + 32, mis)
+    dev.ffill(-7.0, dc)
+    dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+    got = dc.download()
+    assert np.all(got[m * n:] == -7.0)
+    assert parity.frobenius_rel_error(got[:m * n].reshape(m, n), o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+    for t in (da, db, dc):
+        t.free()
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_transpose(dev, seed):
+    rng = np.random.default_rng(6000 + seed)
+    rows, cols = _dims(rng, 2, 900)
+    mis = int(rng.choice([0, 1, 7]))
+    _say("random transpose", seed, (rows, cols), "misalign", mis)
+    x = parity.normal(rng, (rows, cols))
+    dx, dt = dev.array(x, mis), dev.empty(x.size + 32, mis)
+    dev.ffill(-7.0, dt)
+    dev.ftranspose(dx, dt, rows, cols)
+    got = dt.download()
+    assert np.array_equal(got[:x.size].reshape(cols, rows), x.T)
+    assert np.all(got[x.size:] == -7.0)
+    dx.free(); dt.free()
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_conv2d_and_pool(dev, seed):
+    rng = np.random.default_rng(7000 + seed)
+    kh, kw = (int(rng.choice([1, 3, 5, 7, 9])) for _ in range(2))
+    if seed % 5 == 0:
+        kh = kw = int(rng.choice([3, 5]))             # the constant-geometry kernels
+    h = kh - 1 + _dims(rng, 1, 120)[0]
+    w = kw - 1 + _dims(rng, 1, 700)[0]
+    mis = int(rng.choice([0, 5]))
+    _say("random conv2d", seed, (h, w), (kh, kw), "misalign", mis)
+    x, k = parity.normal(rng, (h, w)), parity.normal(rng, (kh, kw))
+    ref = o.fconv2d(x, k)
+    dx, dk, dout = dev.array(x), dev.array(k), dev.empty(ref.size + 32, mis)
+    dev.ffill(-7.0, dout)
+    dev.fconv2d(dx, dk, dout, h, w, kh, kw)
+    got = dout.download()
+    assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+    assert np.all(got[ref.size:] == -7.0)
+    dout.free(); dk.free()
+
+    win = (int(rng.integers(1, min(h, 5) + 1)), int(rng.integers(1, min(w, 5) + 1)))
+    stride = (int(rng.integers(1, 5)), int(rng.integers(1, 5)))
+    _say("random pool", seed, (h, w), win, stride)
+    ref = o.fpool(x, win, stride)
+    dout = dev.empty(ref.size + 32, mis)
+    dev.ffill(-7.0, dout)
+    dev.fpool(dx, dout, h, w, win, stride)
+    got = dout.download()
+    assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+    assert np.all(got[ref.size:] == -7.0)
+    dx.free(); dout.free()
