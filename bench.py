@@ -229,8 +229,10 @@ def bench_transpose(dev, args):
 
 
 def bench_next_builtins(dev, dx, n, args):
-    """frelu / fsoftmax on the sweep's first input, fconv2d 3x3 and fpool 2x2/2 on
-    an 8192 x 8192 image: the builtins the reference has only as generated code."""
+    """flogloss and fmulconcat (the elementwise builtins outside the headline
+    sweep), then the builtins the reference has only as generated code: frelu /
+    fsoftmax on the sweep's first input, fconv2d 3x3 and fpool 2x2/2 on an
+    8192 x 8192 image."""
     out = {}
 
     def report(name, workload, ms, nbytes):
@@ -239,9 +241,18 @@ def bench_next_builtins(dev, dx, n, args):
         out[name] = {"workload": workload, "ms": round(float(np.mean(ms)), 5),
                      "min_ms": round(float(np.min(ms)), 5), "GB/s": round(gbs, 1),
                      "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes": int(nbytes),
-                     "traffic": MEASURED_TRAFFIC_BYTES[name] if n == N_SWEEP else None}
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(name) if n == N_SWEEP else None}
 
     dout = dev.empty(n)
+    # the two elementwise builtins that are not part of the headline sweep
+    rng0 = np.random.default_rng(7)
+    dtruth = dev.array((rng0.random(n, dtype=np.float32) < 0.1).astype(np.float32))
+    dpred = dev.array(rng0.random(n, dtype=np.float32))
+    ms = time_kernel(dev, lambda: dev.flogloss(dpred, dtruth, dout), args.warmup, args.steps)
+    report("flogloss", f"{n} elements, predictions U[0,1), labels Bernoulli(0.1), 2R+1W", ms, 12 * n)
+    ms = time_kernel(dev, lambda: dev.fmulconcat(dtruth, dpred, dout), args.warmup, args.steps)
+    report("fmulconcat", f"{n} elements scaled by gradient[0], 1R+1W", ms, 8 * n)
+    dtruth.free(); dpred.free()
     ms = time_kernel(dev, lambda: dev.frelu(dx, dout), args.warmup, args.steps)
     report("frelu", f"{n} elements, 1R+1W", ms, 8 * n)
     # fsoftmax is three launches (partial sums, total, scale): timed with events around the call
