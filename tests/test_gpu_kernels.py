@@ -384,7 +384,10 @@ def test_conv2d_rejects_even_kernels_and_oversized(dev):
 
 POOL_CASES = [((4, 4), (2, 2), (2, 2)), ((100, 257), (2, 2), (2, 2)), ((101, 333), (3, 3), (2, 2)),
               ((50, 50), (3, 2), (1, 3)), ((64, 64), (64, 64), (1, 1)), ((9, 1000), (1, 1), (1, 1)),
-              ((257, 1031), (2, 2), (2, 2)), ((16, 4100), (4, 4), (4, 4)), ((30, 30), (5, 5), (7, 7))]
+              ((257, 1031), (2, 2), (2, 2)), ((16, 4100), (4, 4), (4, 4)), ((30, 30), (5, 5), (7, 7)),
+              # even widths: the vector-load kernel for non-overlapping 2x2 / 4x4 windows, ragged edges
+              ((101, 334), (2, 2), (2, 2)), ((37, 1030), (2, 2), (2, 2)), ((2, 2), (2, 2), (2, 2)),
+              ((19, 6), (2, 2), (2, 2)), ((9, 516), (4, 4), (4, 4)), ((67, 2052), (4, 4), (4, 4))]
 
 
 @pytest.mark.parametrize("shape,window,stride", POOL_CASES)
