@@ -182,6 +182,7 @@ def main():
         result["next_builtins"] = bench_next_builtins(dev, da, n, args)
         if not args.no_ragged:
             result["ragged"] = bench_ragged(dev, args)
+            result["copies"] = bench_copies(dev)
     da.free(); db.free()
     dev.close()
     dev = None
@@ -282,6 +283,37 @@ def bench_next_builtins(dev, dx, n, args):
     assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
     for t in (dimg, dk, dpool):
         t.free()
+    return out
+
+
+def bench_copies(dev):
+    """Device::copyToDevice / copyToHost as the plugin performs them (pageable host
+    memory): wall time per call including completion, per transfer size."""
+    out = {}
+    for nbytes in (4 << 10, 256 << 10, 4 << 20, 256 << 20):
+        host = np.ones(nbytes // 4, dtype=np.float32)
+        back = np.empty_like(host)
+        buf = dev.empty(nbytes // 4)
+        reps = 5 if nbytes > (64 << 20) else 50
+        for _ in range(2):
+            dev.copy_to_device(buf.ptr, host.ctypes.data, nbytes); dev.copy_to_host(back.ctypes.data, buf.ptr, nbytes)
+        dev.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            dev.copy_to_device(buf.ptr, host.ctypes.data, nbytes)
+        dev.synchronize()
+        up = (time.perf_counter() - t0) / reps
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            dev.copy_to_host(back.ctypes.data, buf.ptr, nbytes)
+        down = (time.perf_counter() - t0) / reps
+        assert back[0] == 1.0 and back[-1] == 1.0
+        label = f"{nbytes >> 10} KiB" if nbytes < (1 << 20) else f"{nbytes >> 20} MiB"
+        out[label] = {"to_device_us": round(up * 1e6, 1), "to_device_GB/s": round(nbytes / up / 1e9, 2),
+                      "to_host_us": round(down * 1e6, 1), "to_host_GB/s": round(nbytes / down / 1e9, 2)}
+        log(f"copy {label:8s}: to device {up * 1e6:9.1f} us ({nbytes / up / 1e9:6.2f} GB/s), "
+            f"to host {down * 1e6:9.1f} us ({nbytes / down / 1e9:6.2f} GB/s)")
+        buf.free()
     return out
 
 
