@@ -45,7 +45,8 @@ SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
 MEASURED_TRAFFIC_BYTES = {
     "fadd": 805290114, "fmul": 805280771, "fdivide": 805292759, "fsigmoid": 536890622,
     "fcopy": 536870912, "ffill": 268459816, "ftranspose": 703813199, "fmatmul": 470152600,
-    "frelu": 536863659, "fsoftmax": 805432513, "fconv2d": 537560171, "fpool": 335545472,
+    "frelu": 536863659, "fsoftmax": 805432513, "fconv2d": 537560171, "fpool": 335573458,
+    "flogloss": 805299755, "fmulconcat": 536858881,
 }
 T_ROWS, T_COLS = 12345, 6789
 MM = 4096
