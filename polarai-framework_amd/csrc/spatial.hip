@@ -135,33 +135,50 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
         if (idx + u * kSegment < total) tile[idx + u * kSegment] = v[u];
     }
   }
+  constexpr int kRegWeights = KH_ != 0 ? KH_ * KW_ : 1;
+  float wreg[kRegWeights];
+  float* const wlds = tile + (kConvRows + KH - 1) * pitch; // generic sizes only
+  if constexpr (KH_ != 0) {
+#pragma unroll
+    for (int i = 0; i < kRegWeights; ++i) wreg[i] = p.weights[i];
+  } else {
+    for (uint32_t i = t; i < KH * KW; i += kSegment) wlds[i] = p.weights[i];
+  }
   __syncthreads();
 
   // A wave takes every fourth row of the band; a lane computes four adjacent
   // outputs of it, so a tap row is read from LDS once for the four and the
-  // wave stores 1 KiB of contiguous, line-aligned output.
-  const uint32_t wave = t / 64, lane = t % 64;
+  // wave stores 1 KiB of contiguous, line-aligned output.  The weights were
+  // fetched before the barrier (registers for the constant sizes, LDS behind
+  // the window otherwise): read through the pointer inside the loop they would
+  // be re-fetched from memory for every row, because the stores may alias them.
+  // The wave index is made a scalar so that everything that depends only on
+  // the row (row shift, row pointers) is computed on the scalar unit.
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t / 64), lane = t % 64;
+  const int32_t xLane = int32_t(ct * kSegment + 4 * lane); // before the row's shift
+  const int32_t ow = int32_t(p.OW);
   for (uint32_t r = wave; r < rowsOut; r += kSegment / 64) {
     const uint32_t y = y0 + r;
     const uint32_t shift = rowShift(y, p.OW, p.outPhase);
-    const int64_t x = int64_t(ct) * kSegment - shift + 4 * lane; // first of the four
-    if (x + 3 < 0 || x >= int64_t(p.OW)) continue;
-    const float* win = tile + r * pitch + (4 * lane + (kLine - 1) - shift);
+    const int32_t x = xLane - int32_t(shift); // first of the four
+    if (x + 3 < 0 || x >= ow) continue;
+    const float* win = tile + r * pitch + (kLine - 1) - shift + 4 * lane;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t a = 0; a < KH; ++a)
       for (uint32_t b = 0; b < KW; ++b) {
-        const float wt = p.weights[a * KW + b];
+        float wt;
+        if constexpr (KH_ != 0) wt = wreg[a * KW_ + b];
+        else wt = wlds[a * KW + b];
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + j] * wt + acc[j];
       }
-    float* dst = p.out + uint64_t(y) * p.OW + x;
-    if (x >= 0 && x + 3 < int64_t(p.OW)) {
-      streamStore(v4f{acc[0], acc[1], acc[2], acc[3]},
-                                  reinterpret_cast<v4f*>(dst));
+    float* const rowOut = p.out + uint64_t(y) * p.OW; // scalar
+    if (x >= 0 && x + 3 < ow) {
+      streamStore(v4f{acc[0], acc[1], acc[2], acc[3]}, reinterpret_cast<v4f*>(rowOut + x));
     } else {
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-        if (x + j >= 0 && x + j < int64_t(p.OW)) dst[j] = acc[j];
+        if (x + j >= 0 && x + j < ow) rowOut[x + j] = acc[j];
     }
   }
 }
@@ -291,8 +308,9 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in, const float* kerne
   p.colTiles = (p.OW + (kLine - 1) + kSegment - 1) / kSegment;
   p.outPhase = phaseOf(out);
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-  const uint64_t ldsBytes = uint64_t(kConvRows + p.KH - 1) *
-                            (kSegment + (kLine - 1) + p.KW - 1) * sizeof(float);
+  const uint64_t ldsBytes = (uint64_t(kConvRows + p.KH - 1) *
+                                 (kSegment + (kLine - 1) + p.KW - 1) +
+                             uint64_t(p.KH) * p.KW) * sizeof(float); // window + weights
   if (ldsBytes <= kMaxConvLds) {
     const uint64_t tiles = uint64_t(p.colTiles) * ((p.OH + kConvRows - 1) / kConvRows);
     POLAR_HIP_REQUIRE(tiles < (1ull << 31) - kXcds, "tensor too large for one launch");
