@@ -14,6 +14,7 @@
 #include "polar_hip.h"
 #include "polar_rt_abi.hpp"
 
+#include <atomic>
 #include <deque>
 #include <mutex>
 
@@ -71,24 +72,27 @@ private:
 
 class HipDevice;
 
-// One point in the stream order of a device.  wait() blocks until the stream
-// has reached it and then runs the callbacks on the calling thread, as the
+// One point in the stream order of a device: the ordinal of a launch on the
+// device's single in-order stream.  No native event is recorded per launch;
+// the first wait() that finds its ordinal not yet known to be complete makes
+// the device record one marker behind everything launched so far and wait for
+// that (HipDevice::waitForLaunch), which completes this event and all earlier
+// ones at once.  wait() then runs the callbacks on the calling thread, as the
 // framework's events do (src/backend/generic/runtime/cuda/CudaEvent.cpp:21-29).
 class HipEvent final : public Event {
 public:
-  HipEvent(HipDevice* device, polar_hip_event* native)
-      : mDevice(device), mNative(native) {}
-  ~HipEvent() override;
+  HipEvent(HipDevice* device, uint64_t launchOrdinal)
+      : mDevice(device), mOrdinal(launchOrdinal) {}
+  ~HipEvent() override = default;
   void wait() override;
   void addCallback(std::function<void()> cb) override;
   auto getDevice() -> Device* override;
 
-  void rearm(polar_hip_event* native);
-  bool idle();
+  void rearm(uint64_t launchOrdinal);
 
 private:
   HipDevice* mDevice;
-  polar_hip_event* mNative; // null once the stream is known to have passed it
+  uint64_t mOrdinal;
   std::mutex mMutex;
   std::vector<std::function<void()>> mCallbacks;
 };
@@ -120,6 +124,9 @@ public:
   void selectBinary(std::vector<std::shared_ptr<ProgramDesc>>& programs) override;
 
   polar_hip_device* native() const { return mDev; }
+  // Returns once launch number `ordinal` (and with it every earlier one) has
+  // completed on the device.
+  void waitForLaunch(uint64_t ordinal);
   float* resolve(BackendAllocator& allocator, const MemoryRecord& record);
 
 private:
@@ -131,6 +138,9 @@ private:
   polar_hip_module* mModule = nullptr;
   std::string mName;
   std::shared_ptr<HipPoolAllocator> mAllocator;
+  std::atomic<uint64_t> mLaunched{0};   // launches enqueued so far
+  std::atomic<uint64_t> mCompleted{0};  // all launches up to this ordinal are known complete
+  std::mutex mSyncMutex;                // one marker in flight at a time
   std::mutex mEventMutex;
   std::deque<std::unique_ptr<HipEvent>> mEvents; // every event ever returned
   std::vector<HipEvent*> mIdleEvents;            // handed back via consumeEvent
