@@ -3,6 +3,8 @@ layouts, transpose, conv2d, pool): small enough for the oracle, awkward enough t
 hit every edge path (sizes around the tile sizes, odd pitches, bases off a line).
 Same bars as the fixed-shape tests: bit-exact for transpose/conv2d/pool, 1e-4
 relative Frobenius for matmul."""
+import os
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,9 @@ import parity
 import polar_oracle as o
 
 pytestmark = pytest.mark.gpu
+
+# more seeds for an occasional longer run: POLAR_RANDOM_SEEDS=10 multiplies the counts below
+SCALE = int(os.environ.get("POLAR_RANDOM_SEEDS", "1"))
 
 
 def _say(*a):
@@ -26,7 +31,7 @@ def _dims(rng, count, hi):
     return out
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(40 * SCALE))
 def test_random_matmul(dev, seed):
     rng = np.random.default_rng(5000 + seed)
     m, n = _dims(rng, 2, 300)
@@ -46,7 +51,7 @@ def test_random_matmul(dev, seed):
         t.free()
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", range(30 * SCALE))
 def test_random_transpose(dev, seed):
     rng = np.random.default_rng(6000 + seed)
     rows, cols = _dims(rng, 2, 900)
@@ -62,7 +67,7 @@ def test_random_transpose(dev, seed):
     dx.free(); dt.free()
 
 
-@pytest.mark.parametrize("seed", range(30))
+@pytest.mark.parametrize("seed", range(30 * SCALE))
 def test_random_conv2d_and_pool(dev, seed):
     rng = np.random.default_rng(7000 + seed)
     kh, kw = (int(rng.choice([1, 3, 5, 7, 9])) for _ in range(2))
