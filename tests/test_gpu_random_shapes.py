@@ -98,3 +98,28 @@ def test_random_conv2d_and_pool(dev, seed):
     assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
     assert np.all(got[ref.size:] == -7.0)
     dx.free(); dout.free()
+
+
+@pytest.mark.parametrize("seed", range(16 * SCALE))
+def test_random_matmul_medium(dev, seed):
+    """Sizes that reach the large tile configurations and the split-K plans; the
+    reference is an fp64 library product (the oracle's sequential fp32 sum is within
+    1e-5 of it at these sizes, and too slow to run for every case)."""
+    rng = np.random.default_rng(8000 + seed)
+    m, n = (int(rng.integers(200, 1600)) for _ in range(2))
+    k = int(rng.integers(64, 3000))
+    if seed % 3 == 0:
+        m, n, k = (v // 4 * 4 for v in (m, n, k))        # the vector-fetch variants
+    if seed % 5 == 0:
+        m, n = (v // 256 * 256 + 256 for v in (m, n)); k = k // 32 * 32 + 32   # edge-free tiles
+    ta, tb = bool(rng.integers(2)), bool(rng.integers(2))
+    _say("random medium matmul", seed, (m, n, k), ta, tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+    da, db, dc = dev.array(a), dev.array(b), dev.empty(m * n)
+    dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+    got = dc.download((m, n))
+    ref = (a.T if ta else a).astype(np.float64) @ (b.T if tb else b).astype(np.float64)
+    assert parity.frobenius_rel_error(got, ref) <= 1e-5
+    for t in (da, db, dc):
+        t.free()
