@@ -48,6 +48,19 @@ int main() {
     CHECK(polar_harness_get_counters(h, &k) == 0);
     CHECK(k.launches == 12 && k.events_waited == 12);
     CHECK(polar_harness_clear_program(h) == 0);
+    // a program handed to the device and a node that names a generated kernel,
+    // integer attributes as 64-bit scalars; the support library's helpers
+    const char image[] = "not a code object: the mock device ignores programs";
+    const char* names[1] = {"gen_kernel"};
+    const uint64_t geometry[6] = {4, 1, 1, 64, 1, 1};
+    CHECK(polar_harness_select_binary(h, 2, "gfx950", image, sizeof(image), 1, names, geometry) == 0);
+    CHECK(polar_harness_select_binary(h, 2, nullptr, nullptr, 0, 0, nullptr, nullptr) == -1);
+    polar_harness_arg gen[3] = {{0, a, 0}, {2, 3, 0}, {0, d, 0}};
+    CHECK(polar_harness_jit_node(h, "gen_kernel", 3, gen, 2) == 0);
+    CHECK(polar_harness_jit_node(h, "", 3, gen, 2) == -1);
+    CHECK(polar_harness_end_cluster(h) == 0);
+    CHECK(polar_harness_run(h) == 0);
+    CHECK(polar_harness_clear_program(h) == 0);
     CHECK(polar_harness_host_write(h, d, data.data(), 128) == 0);
     CHECK(polar_harness_lock(h, d, 0, 0) == 0);
     CHECK(polar_harness_release(h, d, 0) == 0);
