@@ -3,6 +3,7 @@
 // -fsanitize=address,undefined so that lifetime or indexing mistakes in the
 // host code show up without a GPU.
 #include "polar_harness.h"
+#include "polar_rt_support.hpp"
 
 #include <cstdio>
 #include <cstdlib>
@@ -68,6 +69,15 @@ int main() {
     CHECK(out[5] == 1.5f);
     CHECK(polar_harness_raw_device(h) != nullptr && polar_harness_raw_context(h) == nullptr);
     polar_harness_close(h);
+    // construction helpers of the support library
+    uint64_t layout[5];
+    polar_rt_support_graph_handle_layout(layout);
+    CHECK(layout[0] == sizeof(GraphHandle) && layout[1] == 0);
+    auto* allocator = polar_rt_support_allocator_create();
+    auto* host = polar_rt_support_host_device_create();
+    CHECK(allocator != nullptr && host != nullptr && host->getDeviceName() == "host");
+    polar_rt_support_host_device_destroy(host);
+    polar_rt_support_allocator_destroy(allocator);
   }
   std::puts("ok");
   return 0;

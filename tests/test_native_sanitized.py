@@ -15,7 +15,7 @@ def test_harness_under_asan_ubsan(tmp_path):
            "-I" + os.path.join(REPO_ROOT, "include"), "-I" + src,
            os.path.join(REPO_ROOT, "tests", "native", "harness_sanitized.cpp"),
            os.path.join(src, "coherent_allocator.cpp"), os.path.join(src, "support_routines.cpp"),
-           os.path.join(src, "mini_executor.cpp"), "-ldl", "-lpthread", "-o", exe]
+           os.path.join(src, "mini_executor.cpp"), os.path.join(src, "support_factory.cpp"), "-ldl", "-lpthread", "-o", exe]
     subprocess.run(cmd, check=True, capture_output=True, text=True, timeout=300)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0:verify_asan_link_order=0")
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120, env=env)
