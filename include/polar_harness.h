@@ -43,6 +43,8 @@ typedef struct polar_harness_counters {
   uint64_t copies_to_host, bytes_to_host;
   uint64_t events_waited;   /* Event::wait calls made by barriers       */
   uint64_t deferred_releases; /* releases that ran from event callbacks */
+  uint64_t device_name_calls; /* Device::getDeviceName calls on the device
+                                 under test (string work the caller causes) */
 } polar_harness_counters;
 
 /* plugin_path: a runtime plugin to dlopen, or NULL for the built-in CPU mock
@@ -106,6 +108,13 @@ int polar_harness_lock(polar_harness* h, uint64_t vaddr, int device, int lock_ty
 int polar_harness_release(polar_harness* h, uint64_t vaddr, int device);
 int polar_harness_host_write(polar_harness* h, uint64_t vaddr, const float* data,
                              uint64_t count);
+/* Read a tensor the way the framework's OutputNodeAccessor does
+ * (include/polarai/core/node/OutputNodeAccessor.hpp:21-31): through the
+ * allocator's tensor-OBJECT overloads -- lock(tensor, READ_WRITE), get(tensor),
+ * release(tensor) -- with a tensor object of this binary standing for the
+ * framework's TensorInternal. */
+int polar_harness_read_through_tensor_object(polar_harness* h, uint64_t vaddr,
+                                             float* out, uint64_t count);
 
 /* Raw object pointers (Device* of the device under test, the BackendAllocator*,
  * the plugin's Context* or NULL for the mock), for code that wants to use them
@@ -117,7 +126,8 @@ void* polar_harness_raw_context(polar_harness* h);
 
 int polar_harness_get_counters(polar_harness* h, polar_harness_counters* out);
 /* Cap the device layer's capacity (bytes; 0 = no cap) to force the offload
- * path.  Returns -1 if the selected device is not the HIP plugin's. */
+ * path.  Works for the HIP plugin's devices and the built-in mock device;
+ * returns -1 for any other plugin. */
 int polar_harness_set_device_byte_limit(polar_harness* h, uint64_t bytes);
 
 #ifdef __cplusplus

@@ -12,24 +12,87 @@
 //     name string (LayerAllocator.cpp:30-33,60,226-237);
 //   * the offload callback of a device layer really moves the evicted tensor
 //     to RAM (upstream registers one that is never invoked by its layers);
-//   * ath_load hands the loader a flat fp32 view instead of an Accessor
-//     object (see AbstractLoaderInternal below).
+//   * tensors addressed by object (the TensorInternal overloads, which the
+//     framework's OutputNodeAccessor uses to read results --
+//     include/polarai/core/node/OutputNodeAccessor.hpp:21-31) are turned into
+//     records through three member functions of TensorInternal that this
+//     library only declares: they resolve against the framework's polar_core
+//     when the library is linked into it.
 #pragma once
 
 #include "polar_rt_abi.hpp"
 
-// Loader seen by ath_load.  The framework's loaders fill an Accessor<float>
-// over the tensor (include/polarai/core/loader/internal/
-// AbstractLoaderInternal.hpp:32-33); this library passes the flat fp32 view,
-// which is all the framework's MemcpyLoader uses
-// (src/loaders/internal/MemcpyLoaderInternal.cpp:24-27).
-namespace polarai::core::internal {
+#include <initializer_list>
+
+namespace polarai::core {
+// include/polarai/core/tensor/Accessor.hpp:20-44 -- what a loader is handed.
+// Four virtual functions and no virtual destructor, in this order.
+template <typename T> class Accessor {
+public:
+  virtual auto operator()(std::initializer_list<size_t> idx) -> T& = 0;
+  virtual auto operator()(size_t idx) -> T& = 0;
+  virtual auto getShape() -> const std::vector<size_t>& = 0;
+  virtual auto getRawPtr() -> T* = 0;
+
+protected:
+  // first index runs fastest (Accessor.hpp:30-43)
+  auto linearIndex(std::initializer_list<size_t> idx, const std::vector<size_t>& shape) -> size_t {
+    size_t index = 0, stride = 1, d = 0;
+    for (size_t i : idx) {
+      if (d == shape.size()) break;
+      index += i * stride;
+      stride *= shape[d++];
+    }
+    return index;
+  }
+};
+
+namespace internal {
+// include/polarai/core/loader/internal/AbstractLoaderInternal.hpp:26-38.  The
+// framework's class derives from Entity, whose only virtual function is its
+// destructor (include/polarai/core/Entity.hpp:24-43), so a loader's vtable is
+// {destructor, destructor, load}.  This library calls load through that slot
+// and never constructs, destroys, copies or looks inside a loader, so Entity's
+// data members are not restated.
 class AbstractLoaderInternal {
 public:
   virtual ~AbstractLoaderInternal() = default;
-  virtual void load(float* dst, size_t count) = 0;
+  virtual void load(Accessor<float>&) = 0;
 };
-} // namespace polarai::core::internal
+
+// include/polarai/core/tensor/internal/TensorInternal.hpp:25-49.  Only these
+// three members are used (as LayerAllocator.cpp:21-27 does); they are declared,
+// not defined: the definitions are the framework's (src/core/tensor/internal/
+// TensorInternal.cpp).  A tensor object is never created or copied here.
+class TensorInternal {
+public:
+  TensorInternal() = delete;
+  TensorInternal(const TensorInternal&) = delete;
+  DataType getDataType() const;
+  size_t getSize() const;            // number of elements
+  size_t getVirtualAddress() const;  // utils::Index is size_t (utils/Index.hpp:18)
+};
+} // namespace internal
+} // namespace polarai::core
+
+namespace polarai::backend::generic {
+// include/polarai/backend/generic/runtime/BackendAccessor.hpp:23-44 -- the
+// accessor ath_load builds over the tensor's RAM copy (routines.cpp:92-96).
+template <typename T> class BackendAccessor final : public core::Accessor<T> {
+public:
+  BackendAccessor(T* data, size_t dims, uint64_t* shape) : mData(data), mShape(shape, shape + dims) {}
+  auto operator()(std::initializer_list<size_t> idx) -> T& override {
+    return mData[this->linearIndex(idx, mShape)];
+  }
+  auto operator()(size_t idx) -> T& override { return mData[idx]; }
+  auto getShape() -> const std::vector<size_t>& override { return mShape; }
+  auto getRawPtr() -> T* override { return mData; }
+
+private:
+  T* mData;
+  std::vector<size_t> mShape;
+};
+} // namespace polarai::backend::generic
 
 extern "C" {
 // src/backend/generic/runtime/support/api.hpp:18-32

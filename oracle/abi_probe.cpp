@@ -29,6 +29,9 @@
 #include <polarai/backend/generic/runtime/GraphHandle.hpp>
 #include <polarai/backend/generic/runtime/LaunchCommand.h>
 #include <polarai/backend/generic/runtime/TensorInfo.h>
+// header-only in the reference, std headers only: what ath_load hands a loader
+#include <polarai/backend/generic/runtime/BackendAccessor.hpp>
+#include <polarai/core/tensor/Accessor.hpp>
 
 using namespace polarai::backend::generic;
 
@@ -56,17 +59,40 @@ void polar_rt_support_graph_handle_layout(uint64_t out[5]);
 }
 
 namespace {
-// A loader as the support library documents it: a flat fp32 view of the
-// tensor.  `fill` copies data in; `drain` copies the tensor out (how this
-// probe reads results: the library hands the loader the RAM copy).
-struct FlatLoader {
-  virtual ~FlatLoader() = default;
-  virtual void load(float* dst, size_t count) {
-    if (fill != nullptr) std::memcpy(dst, fill, count * sizeof(float));
-    if (drain != nullptr) std::memcpy(drain, dst, count * sizeof(float));
+// A loader with the vtable of the framework's loaders: the virtual destructor
+// inherited from Entity (include/polarai/core/Entity.hpp:29), then
+// load(Accessor<float>&) (include/polarai/core/loader/internal/
+// AbstractLoaderInternal.hpp:32).  AbstractLoaderInternal.hpp itself cannot be
+// included (it needs a cmake-generated export header), but the accessor it is
+// handed is the reference's own class template, so every call below goes
+// through the reference's declaration of Accessor<float>: if the support
+// library built its accessor with another virtual order, these calls would
+// land in the wrong function.  `fill` copies data in; `drain` copies the tensor
+// out (how this probe reads results: the library hands the loader the RAM copy).
+struct ProbeLoader {
+  virtual ~ProbeLoader() = default;
+  virtual void load(polarai::core::Accessor<float>& acc) {
+    const std::vector<size_t>& shape = acc.getShape();
+    size_t count = 1;
+    for (size_t d : shape) count *= d;
+    dims = shape.size();
+    float* raw = acc.getRawPtr();
+    if (fill != nullptr) {
+      std::memcpy(raw, fill, count * sizeof(float));
+      acc(size_t(0)) = fill[0];      // element access by flat index
+      if (dims == 1) acc({count - 1}) = fill[count - 1]; // and by index list
+    }
+    if (drain != nullptr) {
+      std::memcpy(drain, raw, count * sizeof(float));
+      drain[0] = acc(size_t(0));
+      if (dims == 1) drain[count - 1] = acc({count - 1});
+    }
+    ++calls;
   }
   const float* fill = nullptr;
   float* drain = nullptr;
+  size_t dims = 0;
+  int calls = 0;
 };
 } // namespace
 
@@ -205,7 +231,7 @@ int ref_support_evaluate(void* device, uint64_t count, const float* a, const flo
   if (rawAllocator == nullptr || rawHost == nullptr) return 1;
   polar_rt_support_register_device(rawAllocator, dev);
 
-  FlatLoader loadA, loadB, readSum, readA;
+  ProbeLoader loadA, loadB, readSum, readA;
   loadA.fill = a;
   loadB.fill = b;
   readSum.drain = sum;
@@ -274,6 +300,9 @@ int ref_support_evaluate(void* device, uint64_t count, const float* a, const flo
       }
     }
   } // handle (allocator, host device) destroyed
+  if (status == 0 && (loadA.calls != 1 || loadB.calls != 1 || readSum.calls != 1 || readA.calls != 1 ||
+                      loadA.dims != 1))
+    status = 5; // every loader ran exactly once, through the right vtable slot
   return status;
 }
 

@@ -24,7 +24,7 @@ class Arg(C.Structure):
 class Counters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "launches", "copies_to_device", "bytes_to_device", "copies_to_host",
-        "bytes_to_host", "events_waited", "deferred_releases")]
+        "bytes_to_host", "events_waited", "deferred_releases", "device_name_calls")]
 
 
 _vp, _u64, _i = C.c_void_p, C.c_uint64, C.c_int
@@ -49,6 +49,7 @@ SIGNATURES = {
     "polar_harness_lock": (_i, [_vp, _u64, _i, _i]),
     "polar_harness_release": (_i, [_vp, _u64, _i]),
     "polar_harness_host_write": (_i, [_vp, _u64, _vp, _u64]),
+    "polar_harness_read_through_tensor_object": (_i, [_vp, _u64, _vp, _u64]),
     "polar_harness_raw_device": (_vp, [_vp]),
     "polar_harness_raw_allocator": (_vp, [_vp]),
     "polar_harness_raw_context": (_vp, [_vp]),
@@ -295,6 +296,14 @@ class Harness:
     def host_write(self, t, data):
         data = np.ascontiguousarray(data, dtype=np.float32)
         self._ok(self.lib.polar_harness_host_write(self.h, t.vaddr, data.ctypes.data, data.size), "host_write")
+
+    def read_through_tensor_object(self, t):
+        """Read `t` the way the framework's OutputNodeAccessor does: through the
+        allocator's tensor-object overloads."""
+        out = np.empty(t.shape, dtype=np.float32)
+        self._ok(self.lib.polar_harness_read_through_tensor_object(self.h, t.vaddr, out.ctypes.data, out.size),
+                 "read_through_tensor_object")
+        return out
 
     def raw_device(self):
         return self.lib.polar_harness_raw_device(self.h)

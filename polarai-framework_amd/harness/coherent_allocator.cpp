@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 
 namespace polar_harness_detail {
 
@@ -75,20 +76,92 @@ void RamLayer::setTag(MemoryRecord record, size_t tag) {
 
 CoherentAllocator::CoherentAllocator() : mRam(std::make_unique<RamLayer>()) {}
 
+CoherentAllocator::~CoherentAllocator() {
+  for (auto& s : mSlots) forgetDevice(*s.device);
+}
+
+size_t sizeOfDataType(polarai::core::DataType type) {
+  switch (type) {
+  case polarai::core::DataType::DOUBLE: return 8;
+  case polarai::core::DataType::FLOAT: return 4;
+  case polarai::core::DataType::HALF: return 2;
+  default: fatalError(kFatalOther, "Size for dataType is not defined");
+  }
+}
+
+// ---- which devices are "host" -------------------------------------------------
+
 namespace {
-[[noreturn]] void noTensorObjects() {
-  fatalError(kFatalOther, "the mini-executor addresses tensors by record, not by object");
+struct KnownDevice {
+  const Device* object;
+  uintptr_t vtable;
+  bool isHost;
+};
+std::mutex g_knownMutex;
+std::vector<KnownDevice> g_known;
+constexpr size_t kKnownDevicesMax = 64;
+
+uintptr_t vtableOf(const Device& device) {
+  uintptr_t v;
+  std::memcpy(&v, static_cast<const void*>(&device), sizeof(v));
+  return v;
 }
 } // namespace
 
-void CoherentAllocator::allocate(const TensorInternal&) { noTensorObjects(); }
-void CoherentAllocator::deallocate(const TensorInternal&) { noTensorObjects(); }
-void* CoherentAllocator::get(const TensorInternal&) { noTensorObjects(); }
-void CoherentAllocator::lock(const TensorInternal&, LockType) { noTensorObjects(); }
-void CoherentAllocator::release(const TensorInternal&) { noTensorObjects(); }
-void CoherentAllocator::allocate(const TensorInternal&, Device&) { noTensorObjects(); }
-void CoherentAllocator::lock(const TensorInternal&, Device&, LockType) { noTensorObjects(); }
-void* CoherentAllocator::getImpl(const TensorInternal&, Device&) { noTensorObjects(); }
+void rememberDevice(Device& device, bool isHost) {
+  const uintptr_t vt = vtableOf(device);
+  std::scoped_lock g{g_knownMutex};
+  for (auto& k : g_known)
+    if (k.object == &device) {
+      k.vtable = vt;
+      k.isHost = isHost;
+      return;
+    }
+  if (g_known.size() >= kKnownDevicesMax) g_known.erase(g_known.begin());
+  g_known.push_back(KnownDevice{&device, vt, isHost});
+}
+
+void forgetDevice(Device& device) {
+  std::scoped_lock g{g_knownMutex};
+  for (auto it = g_known.begin(); it != g_known.end(); ++it)
+    if (it->object == &device) {
+      g_known.erase(it);
+      return;
+    }
+}
+
+bool isHostDevice(Device& device) {
+  const uintptr_t vt = vtableOf(device);
+  {
+    std::scoped_lock g{g_knownMutex};
+    for (const auto& k : g_known)
+      if (k.object == &device && k.vtable == vt) return k.isHost;
+  }
+  const bool isHost = device.getDeviceName() == "host";
+  rememberDevice(device, isHost);
+  return isHost;
+}
+
+// ---- tensors addressed by object ------------------------------------------------
+
+namespace {
+// LayerAllocator.cpp:21-27 (and the same three lines in every other overload)
+MemoryRecord recordOf(const TensorInternal& tensor) {
+  return MemoryRecord{tensor.getVirtualAddress(),
+                      tensor.getSize() * sizeOfDataType(tensor.getDataType())};
+}
+} // namespace
+
+void CoherentAllocator::allocate(const TensorInternal& t) { allocate(recordOf(t)); }
+void CoherentAllocator::deallocate(const TensorInternal& t) { deallocate(recordOf(t)); }
+void* CoherentAllocator::get(const TensorInternal& t) { return get(recordOf(t)); }
+void CoherentAllocator::lock(const TensorInternal& t, LockType type) { lock(recordOf(t), type); }
+void CoherentAllocator::release(const TensorInternal& t) { release(recordOf(t)); }
+void CoherentAllocator::allocate(const TensorInternal& t, Device& d) { allocate(recordOf(t), d); }
+void CoherentAllocator::lock(const TensorInternal& t, Device& d, LockType type) {
+  lock(recordOf(t), d, type);
+}
+void* CoherentAllocator::getImpl(const TensorInternal& t, Device& d) { return getImpl(recordOf(t), d); }
 
 int CoherentAllocator::slotOf(Device& device) {
   for (size_t i = 0; i < mSlots.size(); ++i)
@@ -120,15 +193,22 @@ void CoherentAllocator::registerDevice(Device& device) {
     s.layer = std::shared_ptr<AllocatorLayerBase>(mRam.get(), [](AllocatorLayerBase*) {});
   }
   Device* dev = &device;
+  // Called by a layer that is about to evict `record`, from inside its
+  // allocate(), which this allocator only calls with mMutex held -- so mState
+  // may be read here.  The device copy is saved only if it is the newest one
+  // and RAM does not have it yet; a stale device copy is simply let go (saving
+  // it would overwrite newer data in RAM and take RAM's tag back with it).
   s.layer->registerMemoryOffloadCallback(
       [this, dev](MemoryRecord record, AllocatorLayerBase& layer) {
-        // called by a layer that evicts `record`: save it to RAM unless RAM
-        // already holds the same version
-        if (mRam->getTag(record) == layer.getTag(record)) return;
+        auto st = mState.find(record.virtualAddress);
+        if (st == mState.end()) return;
+        const size_t version = st->second.version;
+        if (layer.getTag(record) != version || mRam->getTag(record) == version) return;
         if (!mRam->isAllocated(record)) mRam->allocate(record);
         dev->copyToHost(record, mRam->getPtr(record));
-        mRam->setTag(record, layer.getTag(record));
+        mRam->setTag(record, version);
       });
+  rememberDevice(device, s.name == "host");
   mSlots.push_back(std::move(s));
 }
 

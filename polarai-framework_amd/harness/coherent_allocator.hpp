@@ -14,7 +14,7 @@
 //   * copies happen while the allocator's mutex is held, as upstream.
 #pragma once
 
-#include "polar_rt_abi.hpp"
+#include "polar_rt_support.hpp"
 
 #include <list>
 #include <mutex>
@@ -29,6 +29,19 @@ using polarai::core::internal::TensorInternal;
     __attribute__((format(printf, 2, 3)));
 constexpr int kFatalOther = 1;     // ATH_FATAL_OTHER (utils/error/FatalError.hpp:32)
 constexpr int kFatalBadAccess = 4; // ATH_BAD_ACCESS  (utils/error/FatalError.hpp:35)
+
+// include/polarai/core/tensor/DataType.hpp:22-36
+size_t sizeOfDataType(polarai::core::DataType type);
+
+// Is `device` the "host" pseudo-device that input nodes are routed to?  The
+// framework asks the device for its name and compares strings on every
+// support-routine call (routines.cpp:29,40,55).  Here the answer is kept per
+// device object -- keyed by the object's address AND its vtable pointer, so an
+// address reused by an object of another class is not mistaken for the old
+// one -- and only a device seen for the first time is asked for its name.
+bool isHostDevice(Device& device);
+void rememberDevice(Device& device, bool isHost);
+void forgetDevice(Device& device);
 
 // RAM layer: one heap block per record
 // (src/backend/generic/lib/allocators/TrivialAllocator.hpp:23-93).
@@ -57,9 +70,10 @@ private:
 class CoherentAllocator final : public BackendAllocator {
 public:
   CoherentAllocator();
-  ~CoherentAllocator() override = default;
+  ~CoherentAllocator() override;
 
-  // TensorAllocator part: tensor objects never reach the mini-executor
+  // TensorAllocator part: tensors addressed by object; each overload derives
+  // the record from the object (LayerAllocator.cpp:21-27) and forwards
   void allocate(const TensorInternal&) override;
   void deallocate(const TensorInternal&) override;
   void* get(const TensorInternal&) override;

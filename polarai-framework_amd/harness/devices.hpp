@@ -4,9 +4,13 @@
 #pragma once
 
 #include "coherent_allocator.hpp"
+#include "record_layer.hpp"
 
 #include "polar_harness.h"
 
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 namespace polar_harness_detail {
@@ -45,14 +49,38 @@ private:
   std::vector<std::function<void()>> mCallbacks;
 };
 
-// A device with its own memory layer (a second RamLayer standing for device
-// memory) whose launch computes nothing: like the MockDevice of the
+// Block source of the mock device's memory layer: the heap.
+struct HeapBlocks {
+  void* acquire(size_t bytes) {
+    void* p = std::aligned_alloc(64, (bytes + 63) / 64 * 64 + 64);
+    if (p == nullptr) fatalError(kFatalOther, "Failed to allocate RAM memory!");
+    return p;
+  }
+  void give(void* block) { std::free(block); }
+  bool attached() const { return mAttached; }
+  void detach() { mAttached = false; }
+  [[noreturn]] void fail(const char* fmt, ...) __attribute__((format(printf, 2, 3))) {
+    char message[256];
+    va_list ap;
+    va_start(ap, fmt);
+    std::vsnprintf(message, sizeof(message), fmt, ap);
+    va_end(ap);
+    fatalError(kFatalBadAccess, "%s", message);
+  }
+
+private:
+  bool mAttached = true;
+};
+
+// A device with its own memory layer (heap blocks standing for device memory,
+// in the same layer class the GPU plugin uses, so the byte limit and the
+// eviction path work without a GPU) whose launch computes nothing: like the MockDevice of the
 // framework's allocator unit tests (tests/unit/backend/generic/lib/allocators/
 // LayerAllocator.cpp:23-50) it exists so that the coherence protocol and the
 // call sequence can be tested on a machine without a GPU.
 class MockDevice final : public Device {
 public:
-  MockDevice() : mLayer(std::make_shared<RamLayer>()) {}
+  MockDevice() : mLayer(std::make_shared<RecordLayer<HeapBlocks>>()) {}
   DeviceProvider getProvider() const override { return DeviceProvider::HOST; }
   DeviceKind getKind() const override { return DeviceKind::OTHER_ACCELERATOR; }
   std::string getDeviceName() const override { return "mock"; }
@@ -74,10 +102,11 @@ public:
   void consumeEvent(Event* e) override { e->wait(); }
   void selectBinary(std::vector<std::shared_ptr<ProgramDesc>>&) override {}
 
+  void setByteLimit(uint64_t bytes) { mLayer->setByteLimit(bytes); }
   std::vector<std::string> launched;
 
 private:
-  std::shared_ptr<RamLayer> mLayer;
+  std::shared_ptr<RecordLayer<HeapBlocks>> mLayer;
   std::vector<std::unique_ptr<MockEvent>> mEvents;
 };
 
@@ -90,7 +119,10 @@ public:
       : mInner(std::move(inner)), mCounters(c) {}
   DeviceProvider getProvider() const override { return mInner->getProvider(); }
   DeviceKind getKind() const override { return mInner->getKind(); }
-  std::string getDeviceName() const override { return mInner->getDeviceName(); }
+  std::string getDeviceName() const override {
+    mCounters->device_name_calls++;
+    return mInner->getDeviceName();
+  }
   bool isPartitionSupported(PartitionDomain d) override { return mInner->isPartitionSupported(d); }
   bool hasAllocator() override { return mInner->hasAllocator(); }
   std::vector<std::shared_ptr<Device>> partition(PartitionDomain d) override { return mInner->partition(d); }

@@ -22,13 +22,29 @@ public:
   MemcpyLoader(const float* data, size_t count) {
     if (data != nullptr) mData.assign(data, data + count);
   }
-  void load(float* dst, size_t count) override {
+  void load(polarai::core::Accessor<float>& acc) override {
     if (mData.empty()) return;
-    std::memcpy(dst, mData.data(), (count < mData.size() ? count : mData.size()) * sizeof(float));
+    size_t count = 1;
+    for (size_t d : acc.getShape()) count *= d;
+    std::memcpy(acc.getRawPtr(), mData.data(),
+                (count < mData.size() ? count : mData.size()) * sizeof(float));
   }
 
 private:
   std::vector<float> mData;
+};
+
+// What stands for the framework's tensor object in this binary.  The support
+// library only calls three member functions of TensorInternal and leaves them
+// undefined (in a framework build they are polar_core's); here they read this
+// struct, and a HarnessTensor is handed over as a TensorInternal.
+struct HarnessTensor {
+  size_t virtualAddress;
+  polarai::core::DataType type;
+  size_t elements;
+  const polarai::core::internal::TensorInternal& asTensor() const {
+    return *reinterpret_cast<const polarai::core::internal::TensorInternal*>(this);
+  }
 };
 
 struct TensorDecl {
@@ -50,11 +66,22 @@ struct NodeDecl {
 
 } // namespace
 
+namespace polarai::core::internal {
+DataType TensorInternal::getDataType() const {
+  return reinterpret_cast<const HarnessTensor*>(this)->type;
+}
+size_t TensorInternal::getSize() const { return reinterpret_cast<const HarnessTensor*>(this)->elements; }
+size_t TensorInternal::getVirtualAddress() const {
+  return reinterpret_cast<const HarnessTensor*>(this)->virtualAddress;
+}
+} // namespace polarai::core::internal
+
 struct polar_harness {
   void* lib = nullptr;
   Context* ctx = nullptr;
   void (*closeCtx)(Context*) = nullptr;
   int (*setByteLimit)(Device*, uint64_t) = nullptr;
+  MockDevice* mock = nullptr;              // set when the built-in mock device is used
   std::shared_ptr<Device> inner;           // device under test
   std::shared_ptr<CountingDevice> device;  // what the graph code sees
   std::shared_ptr<HostDevice> host;
@@ -84,7 +111,9 @@ int polar_harness_open(const char* plugin_path, int device_index, polar_harness*
   *out = nullptr;
   auto h = std::make_unique<polar_harness>();
   if (plugin_path == nullptr) {
-    h->inner = std::make_shared<MockDevice>();
+    auto mock = std::make_shared<MockDevice>();
+    h->mock = mock.get();
+    h->inner = mock;
     h->deviceCount = 1;
   } else {
     h->lib = dlopen(plugin_path, RTLD_LAZY | RTLD_LOCAL);
@@ -325,6 +354,21 @@ int polar_harness_read(polar_harness* h, uint64_t vaddr, float* out, uint64_t co
   return 0;
 }
 
+// include/polarai/core/node/OutputNodeAccessor.hpp:21-31
+int polar_harness_read_through_tensor_object(polar_harness* h, uint64_t vaddr, float* out,
+                                             uint64_t count) {
+  TensorDecl* t = h ? h->find(vaddr) : nullptr;
+  if (t == nullptr || out == nullptr) return -1;
+  HarnessTensor tensor{static_cast<size_t>(vaddr), polarai::core::DataType::FLOAT, 1};
+  for (uint64_t d : t->shape) tensor.elements *= d;
+  if (count > tensor.elements) return -1;
+  polarai::core::internal::TensorAllocator& allocator = *h->allocator;
+  allocator.lock(tensor.asTensor(), LockType::READ_WRITE);
+  std::memcpy(out, allocator.get(tensor.asTensor()), count * sizeof(float));
+  allocator.release(tensor.asTensor());
+  return 0;
+}
+
 static bool recordOf(polar_harness* h, uint64_t vaddr, MemoryRecord* rec) {
   TensorDecl* t = h ? h->find(vaddr) : nullptr;
   if (t == nullptr) return false;
@@ -382,7 +426,12 @@ int polar_harness_get_counters(polar_harness* h, polar_harness_counters* out) {
 }
 
 int polar_harness_set_device_byte_limit(polar_harness* h, uint64_t bytes) {
-  if (h == nullptr || h->setByteLimit == nullptr) return -1;
+  if (h == nullptr) return -1;
+  if (h->mock != nullptr) {
+    h->mock->setByteLimit(bytes);
+    return 0;
+  }
+  if (h->setByteLimit == nullptr) return -1;
   return h->setByteLimit(h->inner.get(), bytes);
 }
 

@@ -19,9 +19,16 @@ void polar_rt_support_register_device(BackendAllocator* allocator, Device* devic
   allocator->registerDevice(*device);
 }
 
-Device* polar_rt_support_host_device_create() { return new HostDevice(); }
+Device* polar_rt_support_host_device_create() {
+  Device* host = new HostDevice();
+  rememberDevice(*host, true);
+  return host;
+}
 
-void polar_rt_support_host_device_destroy(Device* device) { delete device; }
+void polar_rt_support_host_device_destroy(Device* device) {
+  if (device != nullptr) forgetDevice(*device);
+  delete device;
+}
 
 void polar_rt_support_graph_handle_layout(uint64_t out[5]) {
   out[0] = sizeof(GraphHandle);

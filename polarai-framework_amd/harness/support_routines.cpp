@@ -13,17 +13,13 @@ using namespace polar_harness_detail;
 namespace {
 // src/backend/generic/runtime/utils/utils.hpp:7-17
 MemoryRecord toRecord(const TensorInfo* t) {
-  size_t bytes;
-  switch (static_cast<polarai::core::DataType>(t->dataType)) {
-  case polarai::core::DataType::DOUBLE: bytes = 8; break;
-  case polarai::core::DataType::FLOAT: bytes = 4; break;
-  case polarai::core::DataType::HALF: bytes = 2; break;
-  default: fatalError(kFatalOther, "Size for dataType is not defined");
-  }
+  size_t bytes = sizeOfDataType(static_cast<polarai::core::DataType>(t->dataType));
   for (uint64_t i = 0; i < t->dims; ++i) bytes *= t->shape[i];
   return MemoryRecord{static_cast<size_t>(t->virtAddr), bytes};
 }
-bool isHost(Device& d) { return d.getDeviceName() == "host"; }
+// routines.cpp:29,40,55 compare the device's name with "host" on every call;
+// the answer is looked up per device object instead (no string is built)
+bool isHost(Device& d) { return isHostDevice(d); }
 } // namespace
 
 namespace polar_harness_detail {
@@ -92,7 +88,9 @@ void ath_load(GraphHandle* handle, uint64_t nodeId, TensorInfo* tensor) {
   void* ptr = handle->allocator->get(rec);
   const auto type = static_cast<polarai::core::DataType>(tensor->dataType);
   if (type == polarai::core::DataType::FLOAT) {
-    it->second->load(static_cast<float*>(ptr), rec.allocationSize / 4);
+    // routines.cpp:92-96
+    BackendAccessor<float> acc(static_cast<float*>(ptr), tensor->dims, tensor->shape);
+    it->second->load(acc);
   } else if (type == polarai::core::DataType::DOUBLE) {
     fatalError(kFatalOther, "Double is not supported.");
   }

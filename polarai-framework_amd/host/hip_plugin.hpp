@@ -13,6 +13,7 @@
 
 #include "polar_hip.h"
 #include "polar_rt_abi.hpp"
+#include "record_layer.hpp"
 
 #include <atomic>
 #include <deque>
@@ -23,6 +24,19 @@ namespace polarai::backend::generic::mi355x {
 [[noreturn]] void fatal(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 void checkStatus(int status, const char* what);
 
+// Block source of the GPU's allocator layer: the device library's pool.
+struct PoolBlocks {
+  explicit PoolBlocks(polar_hip_device* dev) : mDev(dev) {}
+  void* acquire(size_t bytes);
+  void give(void* block);
+  bool attached() const { return mDev != nullptr; }
+  void detach() { mDev = nullptr; }
+  [[noreturn]] void fail(const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+private:
+  polar_hip_device* mDev;
+};
+
 // Device-memory layer of one GPU.  Takes the place of the per-tensor raw
 // allocations of the framework's allocator layers
 // (src/backend/generic/runtime/cuda/CudaAllocator.hpp:26-91,
@@ -30,45 +44,7 @@ void checkStatus(int status, const char* what);
 // by virtual address, memory comes from the device library's pool, and the
 // out-of-memory hook is live -- released records are handed to the registered
 // offload callback and then evicted.
-class HipPoolAllocator final : public AllocatorLayerBase {
-public:
-  explicit HipPoolAllocator(polar_hip_device* dev) : mDev(dev) {}
-  ~HipPoolAllocator() override;
-
-  void registerMemoryOffloadCallback(MemoryOffloadCallbackT cb) override;
-  void allocate(MemoryRecord record) override;
-  void deallocate(MemoryRecord record) override;
-  void lock(MemoryRecord record) override;
-  void release(MemoryRecord record) override;
-  void* getPtr(MemoryRecord record) override;
-  bool isAllocated(const MemoryRecord& record) const override;
-  size_t getTag(MemoryRecord record) override;
-  void setTag(MemoryRecord record, size_t tag) override;
-
-  // not part of the interface: capacity limit for tests of the eviction path
-  void setByteLimit(uint64_t bytes) { mByteLimit = bytes; }
-  // called by the owning device just before it closes: frees every block and
-  // turns the layer into an empty shell for owners that outlive the device
-  void detach();
-  uint64_t bytesHeld() const { return mBytesHeld; }
-
-private:
-  struct Entry {
-    void* ptr = nullptr;
-    size_t bytes = 0;
-    size_t tag = 0;
-    bool locked = false;
-    bool released = false;
-  };
-  bool evictOneLocked(std::unique_lock<std::mutex>& guard);
-
-  polar_hip_device* mDev;
-  mutable std::mutex mMutex;
-  std::unordered_map<size_t, Entry> mEntries; // by virtual address
-  MemoryOffloadCallbackT mOffload;
-  uint64_t mByteLimit = 0; // 0 = limited by the device only
-  uint64_t mBytesHeld = 0;
-};
+using HipPoolAllocator = RecordLayer<PoolBlocks>;
 
 class HipDevice;
 

@@ -19,6 +19,12 @@ def available():
 
 
 def load():
+    # The support library inside the probe leaves three member functions of the
+    # framework's TensorInternal undefined (in a framework build they come from
+    # polar_core); the mini-executor's binary defines them for its own tensor
+    # objects, so it is loaded first, with its symbols visible to the probe.
+    from polarai_framework_amd import LIB_HARNESS
+    C.CDLL(LIB_HARNESS, mode=C.RTLD_GLOBAL)
     lib = C.CDLL(LIB)
     lib.ref_struct_layout.argtypes = [C.POINTER(C.c_uint64)]
     lib.ref_context_device_count.argtypes = [C.c_void_p]

@@ -4,6 +4,7 @@
 // host code show up without a GPU.
 #include "polar_harness.h"
 #include "polar_rt_support.hpp"
+#include "devices.hpp"
 
 #include <cstdio>
 #include <cstdlib>
@@ -17,7 +18,49 @@
     }                                                                      \
   } while (0)
 
+// The eviction scan of the allocator layer (the class the GPU plugin's layer is
+// made of, here over heap blocks) with an offload callback that mutates the
+// layer while the scan has dropped its mutex: it locks the victim again, frees
+// other records and adds enough new ones to rehash the table.
+static void evictionScanSurvivesMutatingCallback() {
+  using namespace polar_harness_detail;
+  RecordLayer<HeapBlocks> layer;
+  for (size_t v = 1; v <= 8; ++v) {
+    const MemoryRecord r{v * 100, 64};
+    layer.allocate(r);
+    layer.lock(r);
+    layer.release(r);
+  }
+  layer.setByteLimit(8 * 64);
+  int calls = 0;
+  size_t firstVictim = 0;
+  layer.registerMemoryOffloadCallback([&](MemoryRecord victim, AllocatorLayerBase& l) {
+    if (++calls != 1) return;
+    firstVictim = victim.virtualAddress;
+    l.lock(victim); // taken again while the scan waits
+    int freed = 0;
+    for (size_t v = 1; v <= 8 && freed < 2; ++v)
+      if (v * 100 != victim.virtualAddress) {
+        l.deallocate(MemoryRecord{v * 100, 64});
+        ++freed;
+      }
+    for (size_t v = 0; v < 100; ++v) l.allocate(MemoryRecord{5000 + v, 1}); // rehash
+  });
+  layer.allocate(MemoryRecord{999, 64});
+  CHECK(calls >= 1 && firstVictim != 0);
+  CHECK(layer.isAllocated(MemoryRecord{999, 64}));
+  CHECK(layer.isAllocated(MemoryRecord{firstVictim, 64})); // locked: must not have been evicted
+  CHECK(layer.bytesHeld() <= 8 * 64);
+  // nothing evictable at all: every record locked and the limit reached -> the
+  // scan must end (it reports failure through the fatal path, not tested here)
+  layer.release(MemoryRecord{firstVictim, 64});
+  layer.setByteLimit(0);
+  layer.allocate(MemoryRecord{1000, 64});
+  CHECK(layer.isAllocated(MemoryRecord{1000, 64}));
+}
+
 int main() {
+  evictionScanSurvivesMutatingCallback();
   for (int round = 0; round < 3; ++round) {
     polar_harness* h = nullptr;
     CHECK(polar_harness_open(nullptr, 0, &h) == 0);

@@ -115,6 +115,71 @@ def test_host_write_invalidates_device_copy():
         assert _c(h)["copies_to_host"] == 1
 
 
+def test_results_are_readable_through_tensor_objects():
+    # what the framework's OutputNodeAccessor does: lock(tensor, READ_WRITE), get(tensor),
+    # release(tensor) (include/polarai/core/node/OutputNodeAccessor.hpp:21-31)
+    with harness.Harness(plugin=None) as h:
+        t = h.tensor(2, 3)
+        h.host_write(t, [1, 2, 3, 4, 5, 6])
+        h.lock(t, 0, harness.READ_WRITE); h.release(t, 0)   # the device now holds the newest version
+        before = _c(h)["copies_to_host"]
+        got = h.read_through_tensor_object(t)
+        assert np.array_equal(got.ravel(), [1, 2, 3, 4, 5, 6])
+        assert _c(h)["copies_to_host"] == before + 1          # pulled from the device by the host lock
+        assert np.array_equal(h.read(t).ravel(), got.ravel())
+        h.lock(t, 0, harness.READ_WRITE); h.release(t, 0)   # the lock was released again
+
+
+def test_support_routines_do_no_string_work_after_registration():
+    # upstream compares getDeviceName() with "host" on every ath_allocate / ath_lock /
+    # ath_release (routines.cpp:29,40,55) and keys its tables by the name
+    # (LayerAllocator.cpp:30,60); here a device is asked for its name when it is
+    # registered and never again
+    with harness.Harness(plugin=None) as h:
+        a = h.input(np.arange(8, dtype=np.float32))
+        b = h.input(np.ones(8, dtype=np.float32))
+        h.end_cluster()
+        c = h.fadd(a, 1.0, b, 1.0)
+        h.fmul(c, a)
+        h.end_cluster()
+        h.run()
+        first = _c(h)["device_name_calls"]
+        for _ in range(3):
+            h.run()
+        h.read(c)
+        assert _c(h)["device_name_calls"] == first
+        assert _c(h)["launches"] == 8
+
+
+def test_eviction_of_a_stale_device_copy_keeps_the_newer_host_data():
+    with harness.Harness(plugin=None) as h:
+        t, u = h.tensor(4), h.tensor(4)
+        h.host_write(t, [1, 2, 3, 4])
+        h.lock(t, 0, harness.READ); h.release(t, 0)          # device copy of version 2
+        h.host_write(t, [5, 6, 7, 8])                        # RAM has version 3, device copy is stale
+        h.host_write(u, [9, 9, 9, 9])
+        h.set_device_byte_limit(16)                          # room for one of the two tensors
+        h.lock(u, 0, harness.READ); h.release(u, 0)          # evicts t's stale device copy
+        to_host = _c(h)["copies_to_host"]
+        h.lock(t, 0, harness.READ_WRITE); h.release(t, 0)    # evicts u, uploads RAM's t
+        assert np.array_equal(h.read(t), [5, 6, 7, 8])       # read back from the (mock) device
+        assert _c(h)["copies_to_host"] == to_host + 1        # only the final read; no stale copy was saved
+        assert np.array_equal(h.read(u), [9, 9, 9, 9])
+
+
+def test_eviction_saves_the_only_copy_of_a_result():
+    with harness.Harness(plugin=None) as h:
+        t, u = h.tensor(4), h.tensor(4)
+        h.host_write(t, [1, 2, 3, 4])
+        h.lock(t, 0, harness.READ_WRITE); h.release(t, 0)    # newest version lives on the device only
+        h.host_write(u, [9, 9, 9, 9])
+        h.set_device_byte_limit(16)
+        before = _c(h)["copies_to_host"]
+        h.lock(u, 0, harness.READ); h.release(u, 0)          # evicts t: its device copy must be saved
+        assert _c(h)["copies_to_host"] == before + 1
+        assert np.array_equal(h.read(t), [1, 2, 3, 4])
+
+
 def test_many_read_locks_are_allowed():
     with harness.Harness(plugin=None) as h:
         t = h.tensor(4)
@@ -161,6 +226,15 @@ def test_host_read_write_lock_on_locked_tensor_is_fatal():
     r = _dies("t = h.tensor(4); h.host_write(t, [1,2,3,4]); h.lock(t, 0, 0); h.lock(t, -1, 1)")
     assert r.returncode == 4
     assert "already locked" in r.stderr
+
+
+def test_device_listing_tool_without_gpu():
+    import subprocess
+    from polarai_framework_amd import TOOL_LSPOLAR
+    r = subprocess.run([TOOL_LSPOLAR], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0 and r.stdout.splitlines()[0] == "Total device count: 0"
+    r = subprocess.run([TOOL_LSPOLAR, "/nonexistent/libpolar_rt_hip.so"], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 1 and "Failed to load" in r.stderr
 
 
 def test_plugin_without_devices_is_reported():

@@ -12,7 +12,7 @@ def test_harness_under_asan_ubsan(tmp_path):
     exe = str(tmp_path / "harness_sanitized")
     cmd = ["g++", "-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer",
            "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined",
-           "-I" + os.path.join(REPO_ROOT, "include"), "-I" + src,
+           "-I" + os.path.join(REPO_ROOT, "include"), "-I" + src, "-I" + os.path.join(PACKAGE_DIR, "host"),
            os.path.join(REPO_ROOT, "tests", "native", "harness_sanitized.cpp"),
            os.path.join(src, "coherent_allocator.cpp"), os.path.join(src, "support_routines.cpp"),
            os.path.join(src, "mini_executor.cpp"), os.path.join(src, "support_factory.cpp"), "-ldl", "-lpthread", "-o", exe]
