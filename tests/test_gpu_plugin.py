@@ -12,7 +12,7 @@ import pytest
 
 import parity
 import polar_oracle as o
-from polarai_framework_amd import LIB_PLUGIN, REPO_ROOT, graphs, harness
+from polarai_framework_amd import LIB_PLUGIN, REPO_ROOT, TOOL_LSPOLAR, graphs, harness
 
 pytestmark = pytest.mark.gpu
 
@@ -39,6 +39,18 @@ def test_device_identity(h):
     assert h.device_kind == 1       # DeviceKind::GPU
     name = h.device_name
     assert name != "host" and "gfx950" in name and "hip:0" in name
+
+
+def test_device_listing_tool_reports_what_the_harness_sees(h):
+    # the framework's lspolar for this plugin (utils/lspolar/main.cpp:55-82)
+    _say("lspolar_hip")
+    r = subprocess.run([TOOL_LSPOLAR], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    lines = r.stdout.splitlines()
+    assert lines[0] == f"Total device count: {h.device_count}"
+    names = [l.split(": ", 1)[1] for l in lines if l.startswith("Name       : ")]
+    assert len(names) == h.device_count and h.device_name in names
+    assert "Provider   : HIP" in lines and "Kind       : GPU" in lines and "Allocator  : 1" in lines
 
 
 def _run_case(h, case):
