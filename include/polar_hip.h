@@ -208,6 +208,17 @@ int polar_hip_frelu(polar_hip_device* dev, const float* in, float* out,
  * accumulated in fp64 in a fixed order and rounded to fp32 once. */
 int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out,
                        uint64_t n);
+/* fsoftmax that allocates nothing.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory at the call (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  Same kernels
+ * and same result, bit for bit, as polar_hip_fsoftmax; the partial sums go to
+ * an array in the library's device data segment (256 KiB + 256 B per GPU, held
+ * until the process ends) instead of a pool block.  n is limited to 2^31
+ * elements; more returns POLAR_HIP_ERR_INVALID.  All calls on one GPU share
+ * that array: calls that overlap on one GPU (two host threads, or two devices
+ * handles opened on the same ordinal) race on it. */
+int polar_hip_fsoftmax_static(polar_hip_device* dev, const float* in,
+                              float* out, uint64_t n);
 /* fconv2d: single-channel "valid" correlation, in is height x width, kernel
  * kernelHeight x kernelWidth (odd sizes), out is (height-kernelHeight+1) x
  * (width-kernelWidth+1); fp32 accumulation in tap order (a outer, b inner)

@@ -90,6 +90,7 @@ SIGNATURES = {
                                      C.POINTER(_vp)]),
     "polar_hip_frelu": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fsoftmax": (_i, [_vp, _vp, _vp, _u64]),
+    "polar_hip_fsoftmax_static": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fconv2d": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64]),
     "polar_hip_fpool": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64, _u64]),
     "polar_hip_fmatmul_fsigmoid": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
@@ -300,6 +301,9 @@ class Device:
 
     def fsoftmax(self, x, out, n=None):
         _check(self.lib, self.lib.polar_hip_fsoftmax(self.handle, x.ptr, out.ptr, out.count if n is None else n))
+
+    def fsoftmax_static(self, x, out, n=None):
+        _check(self.lib, self.lib.polar_hip_fsoftmax_static(self.handle, x.ptr, out.ptr, out.count if n is None else n))
 
     def fconv2d(self, x, kernel, out, height, width, kernel_height, kernel_width):
         _check(self.lib, self.lib.polar_hip_fconv2d(self.handle, x.ptr, kernel.ptr, out.ptr, height, width,

@@ -343,7 +343,39 @@ __global__ __launch_bounds__(kSumBlock) void finishSumKernel(const double* parti
   if (threadIdx.x == 0) total[0] = static_cast<float>(t);
 }
 
+// Both passes of fsoftmax with the caller's workspace: `partial` holds one
+// fp64 per work-group of the sum pass, `total` one fp32.  Every slot that is
+// read is written first, so the workspace needs no clearing.
+int softmaxWithWorkspace(polar_hip_device* dev, const float* in, float* out, uint64_t n,
+                         double* partial, float* total) {
+  const uint64_t groups = (n + kSumChunk - 1) / kSumChunk;
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  POLAR_HIP_TRY(launchKernel(dev, expSumKernel, dim3(static_cast<unsigned>(groups)),
+                             dim3(kSumBlock), in, n, partial));
+  POLAR_HIP_TRY(launchKernel(dev, finishSumKernel, dim3(1), dim3(kSumBlock),
+                             static_cast<const double*>(partial), groups, total));
+  return launchEw<SoftmaxScaleOp>(dev, SoftmaxScaleOp{0.0f}, total, in, nullptr, out, n);
+}
+
+// Workspace of polar_hip_fsoftmax_static: lives in the code object's data
+// segment, so every device that loads the library holds its own copy for the
+// life of the process and no call ever allocates.  32768 partials cover 2^31
+// elements (an 8 GiB tensor); 256 KiB + 256 B per device.
+constexpr uint64_t kStaticSoftmaxMaxElements = 1ull << 31;
+constexpr uint64_t kStaticSoftmaxMaxGroups = kStaticSoftmaxMaxElements / kSumChunk;
+static __device__ __align__(256) unsigned char scratch[kStaticSoftmaxMaxGroups * sizeof(double) + 256];
+
 } // namespace
+
+// Called by polar_hip_device_open with the device current: the address of this
+// device's copy of the scratch array.  The array's name is only a host-side
+// handle for this lookup; kernels and copies use the address kept in the device.
+int polar_hip_detail::resolveStaticScratch(polar_hip_device* dev) {
+  void* address = nullptr;
+  POLAR_HIP_TRY(hipGetSymbolAddress(&address, HIP_SYMBOL(scratch)));
+  dev->softmaxScratch = address;
+  return POLAR_HIP_OK;
+}
 
 extern "C" {
 
@@ -425,19 +457,26 @@ int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out, uint6
   int st = polar_hip_alloc(dev, groups * sizeof(double) + sizeof(float), &workspace);
   if (st != POLAR_HIP_OK) return st;
   double* partial = static_cast<double*>(workspace);
-  float* total = reinterpret_cast<float*>(partial + groups);
-  hipError_t e = hipSetDevice(dev->ordinal);
-  if (e == hipSuccess)
-    e = launchKernel(dev, expSumKernel, dim3(static_cast<unsigned>(groups)),
-                     dim3(kSumBlock), in, n, partial);
-  if (e == hipSuccess)
-    e = launchKernel(dev, finishSumKernel, dim3(1), dim3(kSumBlock),
-                     static_cast<const double*>(partial), groups, total);
-  if (e == hipSuccess)
-    st = launchEw<SoftmaxScaleOp>(dev, SoftmaxScaleOp{0.0f}, total, in, nullptr, out, n);
+  st = softmaxWithWorkspace(dev, in, out, n, partial, reinterpret_cast<float*>(partial + groups));
   polar_hip_free(dev, workspace); // stream-ordered: reused only by later work
-  if (e != hipSuccess) return failHip(e, "fsoftmax launch");
   return st;
+}
+
+int polar_hip_fsoftmax_static(polar_hip_device* dev, const float* in, float* out, uint64_t n) {
+  POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  POLAR_HIP_REQUIRE(n == 0 || (in && out), "null tensor");
+  if (n == 0) return POLAR_HIP_OK;
+  if (n > kStaticSoftmaxMaxElements)
+    return fail(POLAR_HIP_ERR_INVALID,
+                "polar_hip_fsoftmax_static: %llu elements exceed the limit of %llu "
+                "(use polar_hip_fsoftmax)",
+                static_cast<unsigned long long>(n),
+                static_cast<unsigned long long>(kStaticSoftmaxMaxElements));
+  POLAR_HIP_REQUIRE(dev->softmaxScratch != nullptr, "the device's scratch array was not resolved");
+  // partials at the start of the array, the total at a fixed place behind them
+  double* partial = static_cast<double*>(dev->softmaxScratch);
+  float* total = reinterpret_cast<float*>(partial + kStaticSoftmaxMaxGroups);
+  return softmaxWithWorkspace(dev, in, out, n, partial, total);
 }
 
 int polar_hip_fsigmoid_flogloss(polar_hip_device* dev, const float* in,

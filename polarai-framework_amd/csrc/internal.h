@@ -48,6 +48,9 @@ struct polar_hip_device {
   polar_hip_event* timeStart = nullptr;
   polar_hip_event* timeStop = nullptr;
 
+  // this device's copy of the file-scope scratch array that
+  // polar_hip_fsoftmax_static works in (resolved once, at open)
+  void* softmaxScratch = nullptr;
 };
 
 struct polar_hip_module {
@@ -63,6 +66,7 @@ namespace polar_hip_detail {
 int fail(polar_hip_status st, const char* fmt, ...)
     __attribute__((format(printf, 2, 3)));
 int failHip(hipError_t e, const char* what);
+int resolveStaticScratch(polar_hip_device* dev); // elementwise.hip
 
 // Every kernel of the library is launched through here.  Normally a plain
 // launch on the device's stream; when a timing pair is armed, the launch

@@ -94,6 +94,12 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
   d->info.l2_bytes = p.l2CacheSize;
   d->info.pci_bus_id = p.pciBusID;
   d->info.hbm_bytes = p.totalGlobalMem;
+  st = resolveStaticScratch(d);
+  if (st != POLAR_HIP_OK) {
+    (void)hipStreamDestroy(d->stream);
+    delete d;
+    return st;
+  }
   *out = d;
   return POLAR_HIP_OK;
 }
