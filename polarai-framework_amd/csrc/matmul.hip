@@ -41,6 +41,7 @@
 // so the result does not depend on scheduling.  Tile shape and split count
 // come from a small cost model (planMatmul) of rounds x k-steps x step time.
 #include "internal.h"
+#include "matmul_epilogue.h"
 
 #include <cmath>
 
@@ -70,28 +71,6 @@ struct MatmulArgs {
   const float* bias;  // M x N, dense (the framework's fadd does not broadcast)
   float scaleAcc, scaleBias;
 };
-
-constexpr int kEpiNone = 0;
-constexpr int kEpiSigmoid = 1;     // sigmoid(acc)
-constexpr int kEpiAddSigmoid = 2;  // sigmoid(scaleAcc*acc + scaleBias*bias)
-
-// The same operations, in the same order, as the separate fadd and fsigmoid
-// kernels apply (sycl/kernels/AddNaive.hpp:33-35, Sigmoid.hpp:32-41), so the
-// fused result is bit-identical to the chain of builtins it replaces.
-__device__ __forceinline__ float applyEpilogue(int epilogue, float acc, const float* bias,
-                                               float scaleAcc, float scaleBias, size_t idx) {
-  if (epilogue == kEpiNone) return acc;
-  float x = acc;
-  if (epilogue == kEpiAddSigmoid) x = scaleAcc * acc + scaleBias * bias[idx];
-  const float eps = 1e-5f;
-  float r = 1.0f / (1.0f + expf(-x));
-  if (fabsf(r - 1.0f) < eps) {
-    r = 1.0f - eps;
-  } else if (fabsf(r) < eps) {
-    r = eps;
-  }
-  return r;
-}
 
 // Fetch of one operand tile (BX x BK) from HBM into registers, and its store
 // into the k-major LDS stage.  KCONTIG: element (x, k) lives at
@@ -500,6 +479,10 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
     return POLAR_HIP_OK;
   }
   const bool ta = transA != 0, tb = transB != 0;
+  // short contraction, one long and one short output dimension: streamed in one
+  // shot per block (matmul_small_k.hip)
+  const MatmulCall call{a, b, c, p.M, p.N, p.K, ta, tb, epilogue, bias, scaleAcc, scaleBias};
+  if (smallKMatmulApplies(call)) return launchSmallKMatmul(dev, call);
   const MatmulPlan plan = planMatmul(p.M, p.N, p.K, dev->info.compute_units);
   switch (plan.config) {
   case 0: return launchTile<256, 256, 32, 4, 4>(dev, ta, tb, p, plan.splits);

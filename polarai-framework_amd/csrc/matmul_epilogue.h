@@ -1,0 +1,50 @@
+// Epilogue of the extended (fused) matmul builtins, shared by every matmul
+// kernel of the library so that a fused call and the chain of builtins it
+// replaces round identically whichever kernel the shape selects.
+#pragma once
+
+#include <cstddef>
+
+namespace polar_hip_detail {
+
+constexpr int kEpiNone = 0;
+constexpr int kEpiSigmoid = 1;     // sigmoid(acc)
+constexpr int kEpiAddSigmoid = 2;  // sigmoid(scaleAcc*acc + scaleBias*bias)
+
+// The same operations, in the same order, as the separate fadd and fsigmoid
+// kernels apply (sycl/kernels/AddNaive.hpp:33-35, Sigmoid.hpp:32-41), so the
+// fused result is bit-identical to the chain of builtins it replaces.
+__device__ __forceinline__ float applyEpilogue(int epilogue, float acc, const float* bias,
+                                               float scaleAcc, float scaleBias, size_t idx) {
+  if (epilogue == kEpiNone) return acc;
+  float x = acc;
+  if (epilogue == kEpiAddSigmoid) x = scaleAcc * acc + scaleBias * bias[idx];
+  const float eps = 1e-5f;
+  float r = 1.0f / (1.0f + expf(-x));
+  if (fabsf(r - 1.0f) < eps) {
+    r = 1.0f - eps;
+  } else if (fabsf(r) < eps) {
+    r = eps;
+  }
+  return r;
+}
+
+// Operands and fused epilogue of one matmul call, as the entry points hand
+// them to a kernel family.
+struct MatmulCall {
+  const float* A;
+  const float* B;
+  float* C;
+  uint32_t M, N, K;
+  bool transA, transB;
+  int epilogue;
+  const float* bias;  // M x N, dense (the framework's fadd does not broadcast)
+  float scaleAcc, scaleBias;
+};
+
+// matmul_small_k.hip: kernels for a short contraction (K <= 128) with one long
+// and one short output dimension.  Returns false if the shape is not theirs.
+bool smallKMatmulApplies(const MatmulCall& call);
+int launchSmallKMatmul(polar_hip_device* dev, const MatmulCall& call);
+
+} // namespace polar_hip_detail

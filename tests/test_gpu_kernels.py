@@ -212,6 +212,43 @@ def test_matmul_unaligned_base(dev, ta, tb):
     assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
 
 
+# short contraction with one long and one short output dimension: the one-shot
+# kernels that keep all of K and of the short dimension in LDS (tall: M long,
+# wide: N long), every layout, ragged edges, K and N that are no multiple of 4/16
+SHORT_K_SHAPES = [(65536, 33, 127), (65536, 127, 33), (33, 65536, 127), (1024, 1, 1), (1031, 16, 4),
+                  (2049, 17, 128), (1, 1024, 5), (128, 3001, 100), (1500, 128, 77), (4096, 48, 64),
+                  (100, 1111, 3), (7000, 65, 2)]
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("mnk", SHORT_K_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_short_contraction_tall_and_wide(dev, ta, tb, mnk):
+    m, n, k = mnk
+    _say("short-k matmul", ta, tb, mnk)
+    rng = np.random.default_rng(m * 7 + n * 1009 + k + 2 * ta + tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    o.set_threads(o.hw_threads())
+    try:
+        # small integers: exact in fp32 in any order, so a wrong index shows as a wrong value
+        a = rng.integers(-8, 9, sa).astype(np.float32)
+        b = rng.integers(-8, 9, sb).astype(np.float32)
+        da, db, dc = dev.array(a, 1), dev.array(b, 3), dev.empty(m * n + 64, 2)
+        dev.ffill(-7.0, dc, m * n + 64)
+        dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+        got = dc.download()
+        assert np.array_equal(got[:m * n].reshape(m, n), o.fmatmul(ta, tb, a, b))
+        assert np.all(got[m * n:] == -7.0)                 # nothing written past the end
+        for t in (da, db, dc):
+            t.free()
+        a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+        got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+        assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+        assert np.array_equal(got, _matmul_device(dev, ta, tb, a, b, m, n, k))   # repeatable
+    finally:
+        o.set_threads(1)
+
+
 SPLIT_K_SHAPES = [(33, 127, 4099), (33, 127, 65536), (256, 10, 784), (10, 256, 2051), (64, 64, 8192),
                   (130, 70, 3000), (1024, 1024, 4096)]
 
@@ -409,7 +446,8 @@ def test_pool_bit_exact(dev, shape, window, stride):
 
 # ---- extended (fused) builtins ----------------------------------------------------
 
-FUSED_SHAPES = [(256, 10, 784), (64, 64, 64), (33, 127, 4096), (300, 257, 129), (1024, 1024, 512), (5, 3, 0)]
+FUSED_SHAPES = [(256, 10, 784), (64, 64, 64), (33, 127, 4096), (300, 257, 129), (1024, 1024, 512), (5, 3, 0),
+                (2050, 33, 127), (40, 1500, 30)]
 
 
 @pytest.mark.parametrize("mnk", FUSED_SHAPES)
