@@ -14,8 +14,8 @@
 // The next tile is fetched into registers while the current one is multiplied
 // (two LDS stages, one barrier per step).  Each wave owns a (BM/WM) x (BN/WN)
 // sub-tile as TM x TN accumulator blocks of 32x32; per k-pair it reads TM + TN
-// LDS words per lane and issues TM*TN MFMAs.  LDS row pitch is BX + 4 words so
-// the scattered stores of the k-contiguous case spread over the banks.
+// LDS words per lane and issues TM*TN MFMAs.  The LDS row pitch is chosen per
+// operand so that neither the fill nor the fragment reads collide on banks.
 //
 // What bounds the 4096^3 case on MI355X (measured): the matrix pipes need 2^31
 // busy cycles over 1024 SIMDs; under this kernel's LDS and L2 traffic the chip
@@ -53,7 +53,14 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int kLdsPad = 4;
+// LDS row pitch of a BX-wide operand stage.  A stage that is filled by 16-byte
+// writes (operand contiguous along x) needs a pitch that is a multiple of 4
+// words; BX + 4 also puts the two rows a wave reads per fragment four banks
+// apart.  A stage that is filled by scattered single words (operand contiguous
+// along k: a lane writes 4 consecutive k of one x, i.e. 4 rows) gets an odd
+// pitch: within a half-wave the 8 rows and 4 columns written by one instruction
+// then fall on 32 different banks (with BX + 4 they fell on 8).
+template <int BX, bool KCONTIG> constexpr int ldsPitch() { return BX + (KCONTIG ? 1 : 4); }
 constexpr int kXcds = 8;
 
 struct MatmulArgs {
@@ -130,7 +137,7 @@ struct TileFetch {
   }
 
   __device__ __forceinline__ void store(float* S, int t) const {
-    constexpr int LD = BX + kLdsPad;
+    constexpr int LD = ldsPitch<BX, KCONTIG>();
     if constexpr (VEC) {
 #pragma unroll
       for (int v = 0; v < kVecs; ++v) {
@@ -182,7 +189,7 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int LDA = BM + kLdsPad, LDB = BN + kLdsPad;
+  constexpr int LDA = ldsPitch<BM, !TA>(), LDB = ldsPitch<BN, TB>();
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile is made of 32x32");
   static_assert(BK % 4 == 0, "BK multiple of 4");
 
