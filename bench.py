@@ -110,6 +110,8 @@ def main():
     ap.add_argument("--no-matmul", action="store_true", help="skip the matmul/transpose legs")
     ap.add_argument("--no-ragged", action="store_true",
                     help="skip the ragged-shape leg (keeps a profile to one problem size per kernel)")
+    ap.add_argument("--no-probes", action="store_true",
+                    help="skip the memory-pattern probes (pattern ceilings measured beside the builtins)")
     ap.add_argument("--no-graphs", action="store_true",
                     help="skip the model-graph legs (keeps a profile to one problem size per kernel)")
     args = ap.parse_args()
@@ -222,6 +224,8 @@ def main():
     da.free(); db.free()
     dev.close()
     dev = None
+    if not args.no_probes:
+        result["ceilings"] = bench_ceilings(args, n)
     if not args.no_graphs:
         result["graphs"] = bench_graphs()
 
@@ -363,6 +367,70 @@ def bench_next_builtins(dev, dx, n, args):
     assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
     for t in dimgs + dpools + [dk]:
         t.free()
+    return out
+
+
+def bench_ceilings(args, n):
+    """Memory-pattern probes (kernels that move a builtin's bytes in its pattern
+    and do none of its work) timed in this run on this GPU: what HBM delivers
+    for streams of reads and writes in the ratios the builtins have, and for the
+    reads and writes of a tiled transpose of the benchmark's matrix."""
+    import ctypes as C
+    from polarai_framework_amd import LIB_PROBES
+    lib = C.CDLL(LIB_PROBES)
+    reps, warm = max(10, args.steps), max(2, args.warmup)
+    us = (C.c_float * reps)()
+
+    def run(fn, *a):
+        status = fn(*a, ROTATE, warm, reps, us)
+        if status != 0:
+            raise RuntimeError(f"{fn.__name__} failed with hipError {status}")
+        return float(np.mean(list(us)))
+
+    lib.polar_probe_streams.argtypes = [C.c_int, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
+    lib.polar_probe_read.argtypes = [C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
+    lib.polar_probe_transpose_pattern.argtypes = [C.c_uint32, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int,
+                                                  C.c_int, C.POINTER(C.c_float)]
+    out = {"note": "probe kernels, not builtins: same bytes and pattern, no work; back-to-back launches, "
+                   f"{ROTATE} buffer sets in rotation", "streams": {}, "read_only": {}, "transpose_pattern": {}}
+    for reads, like in ((0, "ffill"), (1, "fcopy frelu fsigmoid fconv2d"), (2, "fadd fmul fdivide flogloss"),
+                        (4, "fpool 2x2 (4 reads per write)")):
+        for ranges in (0, 1):
+            t = run(lib.polar_probe_streams, reads, n, ranges)
+            gbs = 4 * n * (reads + 1) / (t * 1e-6) / 1e9
+            order = "a contiguous eighth per XCD" if ranges else "pieces dealt round-robin to the XCDs"
+            out["streams"][f"{reads}R+1W, {order}"] = {"us": round(t, 2), "GB/s": round(gbs, 1),
+                                                       "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                                                       "pattern_of": like}
+            log(f"probe {reads}R+1W streams, {order}: {t:7.1f} us  {gbs:7.1f} GB/s  "
+                f"{100 * gbs / HBM_PEAK_GBS:5.1f}%   ({like})")
+    for unroll in (2, 4, 8, 16):
+        t = run(lib.polar_probe_read, n, unroll)
+        gbs = 4 * n / (t * 1e-6) / 1e9
+        out["read_only"][f"{unroll} x 16 B per lane"] = {"us": round(t, 2), "GB/s": round(gbs, 1),
+                                                         "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        log(f"probe read only, {unroll:2d} loads per lane: {t:7.1f} us  {gbs:7.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}%")
+    best = max(out["read_only"].values(), key=lambda v: v["GB/s"])
+    out["read_only"]["best_GB/s"] = best["GB/s"]
+    names = {0: "32x256 tile, 1024 lanes", 1: "32x128 tile, 512 lanes", 2: "32x128 tile, 256 lanes",
+             3: "64x256 tile, 1024 lanes", 4: "32x64 tile, 256 lanes"}
+    orders = {0: "row tiles fastest", 1: "column tiles fastest", 2: "column-tile range per XCD"}
+    nbytes = 8 * T_ROWS * T_COLS
+    for variant in names:
+        for order in orders:
+            t = run(lib.polar_probe_transpose_pattern, T_ROWS, T_COLS, variant, order)
+            gbs = nbytes / (t * 1e-6) / 1e9
+            out["transpose_pattern"][f"{names[variant]}, {orders[order]}"] = {
+                "us": round(t, 2), "GB/s": round(gbs, 1), "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+            log(f"probe transpose pattern {names[variant]}, {orders[order]}: {t:7.1f} us  {gbs:7.1f} GB/s  "
+                f"{100 * gbs / HBM_PEAK_GBS:5.1f}%")
+    best = max(out["transpose_pattern"].values(), key=lambda v: v["GB/s"])
+    out["transpose_pattern"]["best_GB/s"] = best["GB/s"]
+    # the plain copy of the transpose's byte count
+    nt = (T_ROWS * T_COLS) // 4 * 4
+    t = run(lib.polar_probe_streams, 1, nt, 0)
+    out["copy_of_transpose_bytes"] = {"us": round(t, 2), "GB/s": round(8 * nt / (t * 1e-6) / 1e9, 1)}
+    log(f"probe copy of {8 * nt} bytes: {t:7.1f} us  {8 * nt / (t * 1e-6) / 1e9:7.1f} GB/s")
     return out
 
 

@@ -293,11 +293,37 @@ int launchEw(polar_hip_device* dev, const Op& op, const float* scalarSrc,
 // ---- fsoftmax, first pass: total = sum exp(x) over the whole tensor ----------
 // Work-group g sums elements [g*kSumChunk, (g+1)*kSumChunk) into partial[g];
 // lanes and partials accumulate in fp64 (groups of four terms in fp32 first)
-// and every order is fixed by the index,
-// so the result does not depend on scheduling.  Plain (temporal) loads: the
+// and every order is fixed by the index, so the result does not depend on
+// scheduling.  A second, single-group launch adds up the partials: letting the
+// group that finishes last do it inside the first launch needs a device-wide
+// release per group, and the L2 write-back that implements it doubled the
+// pass's duration (48 -> 94 us on 2^26 elements).  Plain (temporal) loads: the
 // second pass reads the tensor again and should find it in cache if it fits.
 constexpr int kSumBlock = 256;
 constexpr uint64_t kSumChunk = 65536; // elements per work-group
+constexpr int kSumBatch = 8;          // 16-byte loads a lane has in flight while it works on the previous 8
+constexpr int kSumRounds = kSumChunk / 4 / kSumBlock / kSumBatch;
+static_assert(kSumRounds * kSumBatch * kSumBlock * 4 == kSumChunk, "chunk is whole rounds");
+
+// exp(x) for the terms of the sum: 2^n * 2^r with n = round(x log2 e) and
+// r = x log2 e - n in [-0.5, 0.5] computed with two fused multiply-adds (log2 e
+// split into a high and a low part), the hardware's exp2 for 2^r and ldexp for
+// the scaling, which also produces the overflow to infinity and the underflow
+// to zero.  7 instructions instead of the 13 of the library's expf (which
+// spends the difference on range checks that the clamp below replaces); with
+// them the pass was bound by instruction issue, not by memory.  The error is
+// below 1.5 units in the last place; the total only enters the result through
+// its fp32 rounding.  NaN stays NaN; the clamp keeps x log2 e inside the
+// integer range (exp overflows above 88.73 and is 0 below -103.98 anyway).
+__device__ __forceinline__ float expTerm(float x) {
+  const float kLog2eHi = 1.44269502162933349609375f; // fp32 nearest to log2 e
+  const float kLog2eLo = 1.925963033500011e-8f;      // log2 e - kLog2eHi
+  x = __builtin_amdgcn_fmed3f(x, -104.0f, 89.0f);
+  const float n = __builtin_rintf(x * kLog2eHi);
+  float r = __builtin_fmaf(x, kLog2eHi, -n);
+  r = __builtin_fmaf(x, kLog2eLo, r);
+  return __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(n));
+}
 
 __device__ __forceinline__ double blockSum(double v, double* lds) {
 #pragma unroll
@@ -318,16 +344,29 @@ __global__ __launch_bounds__(kSumBlock) void expSumKernel(const float* x, uint64
   const uint64_t end = begin + kSumChunk < n ? begin + kSumChunk : n;
   double acc = 0.0;
   if ((reinterpret_cast<uintptr_t>(x) & 15u) == 0 && end - begin == kSumChunk) {
-    const v4f* x4 = reinterpret_cast<const v4f*>(x + begin);
-#pragma unroll 8
-    for (uint32_t i = threadIdx.x; i < kSumChunk / 4; i += kSumBlock) {
-      const v4f v = x4[i];
-      // four terms are added in fp32 (two roundings, 1.2e-7 relative at worst),
-      // everything above that in fp64
-      acc += double((expf(v.x) + expf(v.y)) + (expf(v.z) + expf(v.w)));
+    const v4f* x4 = reinterpret_cast<const v4f*>(x + begin) + threadIdx.x;
+    // the loads of round r+1 are issued before the exponentials of round r, so
+    // a wave has memory requests in flight while it computes
+    v4f v[2][kSumBatch];
+#pragma unroll
+    for (int u = 0; u < kSumBatch; ++u) v[0][u] = x4[u * kSumBlock];
+#pragma unroll
+    for (int r = 0; r < kSumRounds; ++r) {
+      if (r + 1 < kSumRounds) {
+#pragma unroll
+        for (int u = 0; u < kSumBatch; ++u)
+          v[(r + 1) & 1][u] = x4[((r + 1) * kSumBatch + u) * kSumBlock];
+      }
+#pragma unroll
+      for (int u = 0; u < kSumBatch; ++u) {
+        const v4f e = v[r & 1][u];
+        // four terms are added in fp32 (two roundings, 1.2e-7 relative at worst),
+        // everything above that in fp64
+        acc += double((expTerm(e.x) + expTerm(e.y)) + (expTerm(e.z) + expTerm(e.w)));
+      }
     }
   } else {
-    for (uint64_t i = begin + threadIdx.x; i < end; i += kSumBlock) acc += double(expf(x[i]));
+    for (uint64_t i = begin + threadIdx.x; i < end; i += kSumBlock) acc += double(expTerm(x[i]));
   }
   const double total = blockSum(acc, lds);
   if (threadIdx.x == 0) partial[blockIdx.x] = total;
@@ -452,14 +491,14 @@ int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out, uint6
   if (n == 0) return POLAR_HIP_OK;
   const uint64_t groups = (n + kSumChunk - 1) / kSumChunk;
   POLAR_HIP_REQUIRE(groups < (1ull << 31), "tensor too large for one launch");
-  // workspace: one fp64 partial per work-group, then the fp32 total
-  void* workspace = nullptr;
-  int st = polar_hip_alloc(dev, groups * sizeof(double) + sizeof(float), &workspace);
+  // one fp64 partial per work-group in the device's workspace, the fp32 total
+  // behind them
+  std::lock_guard<std::mutex> g(dev->workspaceMu);
+  void* area = nullptr;
+  const int st = workspaceFor(dev, groups * sizeof(double) + sizeof(float), &area);
   if (st != POLAR_HIP_OK) return st;
-  double* partial = static_cast<double*>(workspace);
-  st = softmaxWithWorkspace(dev, in, out, n, partial, reinterpret_cast<float*>(partial + groups));
-  polar_hip_free(dev, workspace); // stream-ordered: reused only by later work
-  return st;
+  double* partial = static_cast<double*>(area);
+  return softmaxWithWorkspace(dev, in, out, n, partial, reinterpret_cast<float*>(partial + groups));
 }
 
 int polar_hip_fsoftmax_static(polar_hip_device* dev, const float* in, float* out, uint64_t n) {

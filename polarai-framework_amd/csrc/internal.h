@@ -51,6 +51,17 @@ struct polar_hip_device {
   // this device's copy of the file-scope scratch array that
   // polar_hip_fsoftmax_static works in (resolved once, at open)
   void* softmaxScratch = nullptr;
+
+  // Workspace of the builtins that run more than one kernel per call (softmax
+  // partial sums, split-K partial products).  Allocated when the device is
+  // opened, so a launch neither allocates nor waits; a call that needs more
+  // replaces it by one twice as large, and the outgrown block stays until the
+  // device is closed because kernels already enqueued may still use it.
+  // workspaceMu is held while a call enqueues the kernels that share it.
+  std::mutex workspaceMu;
+  void* workspace = nullptr;
+  uint64_t workspaceBytes = 0;
+  std::vector<void*> outgrownWorkspaces;
 };
 
 struct polar_hip_module {
@@ -67,6 +78,12 @@ int fail(polar_hip_status st, const char* fmt, ...)
     __attribute__((format(printf, 2, 3)));
 int failHip(hipError_t e, const char* what);
 int resolveStaticScratch(polar_hip_device* dev); // elementwise.hip
+
+constexpr uint64_t kInitialWorkspace = 64ull << 20;
+// *area: at least `bytes` of device memory, 256-byte aligned, contents
+// undefined.  Caller holds dev->workspaceMu.  Allocates only when `bytes`
+// exceeds what the device holds.
+int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area); // runtime.hip
 
 // Every kernel of the library is launched through here.  Normally a plain
 // launch on the device's stream; when a timing pair is armed, the launch
@@ -101,7 +118,12 @@ inline hipError_t launchKernel(polar_hip_device* dev, void (*kernel)(KArgs...),
 // with both (stores without any hint 88 us).
 typedef float polar_v4f __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void streamStore(polar_v4f value, polar_v4f* address) {
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt" : : "v"(address), "v"(value) : "memory");
+  // The compiler does not look into the asm text, so it cannot see that a
+  // 128-bit store's data registers must not be overwritten by the next
+  // instruction or two (the hazard it pads itself for stores it emits): the
+  // two wait states are part of the statement.
+  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1"
+               : : "v"(address), "v"(value) : "memory");
 }
 __device__ __forceinline__ void streamStore(float value, float* address) {
   asm volatile("global_store_dword %0, %1, off sc1 nt" : : "v"(address), "v"(value) : "memory");

@@ -382,10 +382,15 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
   const bool edge = p.M % BM != 0 || p.N % BN != 0 || p.K % BK != 0;
 
   float* const c = p.C;
-  void* workspace = nullptr;
   const uint64_t count = uint64_t(p.M) * p.N;
+  // partial products go to the device's workspace; the lock keeps another
+  // thread's call from enqueuing its own user of the workspace between this
+  // call's two kernels
+  std::unique_lock<std::mutex> workspaceLock(dev->workspaceMu, std::defer_lock);
+  void* workspace = nullptr;
   if (splits > 1) {
-    int st = polar_hip_alloc(dev, count * splits * sizeof(float), &workspace);
+    workspaceLock.lock();
+    int st = workspaceFor(dev, count * splits * sizeof(float), &workspace);
     if (st != POLAR_HIP_OK) return st;
     p.C = static_cast<float*>(workspace);
   }
@@ -394,14 +399,9 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
   else if (!ta && tb) st = launchLayout<BM, BN, BK, WM, WN, false, true>(dev, p, vec, edge);
   else if (ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, true, false>(dev, p, vec, edge);
   else st = launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
-  if (splits > 1) {
-    if (st == POLAR_HIP_OK) {
-      hipError_t e = launchReduce(dev, static_cast<const float*>(workspace), c, count, splits, p);
-      if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
-    }
-    // stream-ordered pool: the block may be handed out again only to work
-    // enqueued after the reduction
-    polar_hip_free(dev, workspace);
+  if (splits > 1 && st == POLAR_HIP_OK) {
+    hipError_t e = launchReduce(dev, static_cast<const float*>(workspace), c, count, splits, p);
+    if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
   }
   return st;
 }

@@ -38,6 +38,24 @@ int failHip(hipError_t e, const char* what) {
   return fail(st, "%s failed: %s (%d)", what, hipGetErrorString(e),
               static_cast<int>(e));
 }
+
+// ---- workspace ----------------------------------------------------------------
+
+int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area) {
+  if (bytes > dev->workspaceBytes) {
+    uint64_t wanted = dev->workspaceBytes ? dev->workspaceBytes : kInitialWorkspace;
+    while (wanted < bytes) wanted *= 2;
+    POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+    void* block = nullptr;
+    POLAR_HIP_TRY(hipMalloc(&block, wanted));
+    if (dev->workspace) dev->outgrownWorkspaces.push_back(dev->workspace);
+    dev->workspace = block;
+    dev->workspaceBytes = wanted;
+  }
+  *area = dev->workspace;
+  return POLAR_HIP_OK;
+}
+
 } // namespace polar_hip_detail
 
 using namespace polar_hip_detail;
@@ -95,6 +113,11 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
   d->info.pci_bus_id = p.pciBusID;
   d->info.hbm_bytes = p.totalGlobalMem;
   st = resolveStaticScratch(d);
+  if (st == POLAR_HIP_OK) {
+    std::lock_guard<std::mutex> g(d->workspaceMu);
+    void* unused = nullptr;
+    st = polar_hip_detail::workspaceFor(d, polar_hip_detail::kInitialWorkspace, &unused);
+  }
   if (st != POLAR_HIP_OK) {
     (void)hipStreamDestroy(d->stream);
     delete d;
@@ -111,6 +134,8 @@ int polar_hip_device_close(polar_hip_device* dev) {
   for (auto& kv : dev->cached)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : dev->live) (void)hipFree(kv.first);
+  if (dev->workspace) (void)hipFree(dev->workspace);
+  for (void* p : dev->outgrownWorkspaces) (void)hipFree(p);
   for (auto* e : dev->allEvents) {
     (void)hipEventDestroy(e->ev);
     delete e;

@@ -16,12 +16,27 @@
 //    there; the accumulation is the reference's: fp32, a outer / b inner,
 //    product rounded before the add (the file is compiled with
 //    -ffp-contract=off).  3x3 and 5x5 are compiled with constant bounds.
+//    Measured on an 8192^2 image, 3x3, buffers rotated (537 MB per launch; a
+//    plain copy of that size takes 80 us): 93 us.  HBM traffic is 1.002 x the
+//    algorithmic bytes and the LDS reads are free of bank conflicts; the
+//    counters show the waves parked at the barrier, waiting for the window,
+//    for most of their life.  Shapes that measured slower than this one: four
+//    adjacent outputs per lane with one 16-byte store (115 us with the window
+//    row-major, 111 us with the window kept as four interleaved quarters so
+//    that the reads stay conflict-free, 16-byte staging loads), no LDS at all
+//    (a lane fetching its own KW+3 inputs per tap row: 98-110 us), a resident
+//    grid of groups that prefetch their next band into registers while they
+//    compute (116 us in row-major band order, 152 us walking down strips),
+//    16 or more rows per band (96-115 us); 8 to 12 rows measure the same.
 //  * fpool reads its windows straight from memory: with stride >= window each
 //    input element is used once, and the lanes of a wave walk consecutive
 //    windows, so the lines they touch are consumed completely by that wave.
 //    Non-overlapping 2x2 and 4x4 windows have a kernel of their own that takes
-//    a window row per vector load and issues a whole band's loads at once
-//    (8192^2, 2x2: 58 -> 47.5 us).
+//    a window row per vector load and issues a whole band's loads at once.
+//    Short bands are better (8192^2, 2x2, buffers rotated: 61.7 / 55.7 / 57.1 /
+//    58.7 / 60.3 us for 1 / 2 / 4 / 8 / 16 rows per group; four input streams
+//    merged into one output stream at full vector width take 54 us for the
+//    same bytes).
 #include "internal.h"
 
 using namespace polar_hip_detail;
@@ -32,8 +47,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kSegment = 256; // output columns per work-group = lanes
 constexpr int kLine = 32;     // floats per 128-byte line
-constexpr int kConvRows = 16; // output rows per fconv2d work-group
-constexpr int kPoolRows = 8;  // output rows per fpool work-group
+constexpr int kConvRows = 12; // output rows per fconv2d work-group
+constexpr int kPoolRows = 2;  // output rows per fpool work-group
 constexpr uint32_t kMaxConvLds = 64 * 1024;
 
 // Work-group id -> tile index such that each XCD (ids equal modulo 8 share
@@ -146,23 +161,25 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   }
   __syncthreads();
 
-  // A wave takes every fourth row of the band; a lane computes four adjacent
-  // outputs of it, so a tap row is read from LDS once for the four and the
-  // wave stores 1 KiB of contiguous, line-aligned output.  The weights were
+  // A wave takes every fourth row of the band; a lane computes the four
+  // outputs lane, lane+64, lane+128, lane+192 of the row's segment, so the
+  // lanes of a wave read consecutive LDS words for every tap (no bank
+  // conflicts: four adjacent outputs per lane would put the lanes 4 words
+  // apart, on 8 of the 32 banks) and each of the wave's four stores covers two
+  // whole 128-byte lines.  The weights were
   // fetched before the barrier (registers for the constant sizes, LDS behind
   // the window otherwise): read through the pointer inside the loop they would
   // be re-fetched from memory for every row, because the stores may alias them.
   // The wave index is made a scalar so that everything that depends only on
   // the row (row shift, row pointers) is computed on the scalar unit.
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t / 64), lane = t % 64;
-  const int32_t xLane = int32_t(ct * kSegment + 4 * lane); // before the row's shift
+  const int32_t xLane = int32_t(ct * kSegment + lane); // before the row's shift
   const int32_t ow = int32_t(p.OW);
   for (uint32_t r = wave; r < rowsOut; r += kSegment / 64) {
     const uint32_t y = y0 + r;
     const uint32_t shift = rowShift(y, p.OW, p.outPhase);
-    const int32_t x = xLane - int32_t(shift); // first of the four
-    if (x + 3 < 0 || x >= ow) continue;
-    const float* win = tile + r * pitch + (kLine - 1) - shift + 4 * lane;
+    const int32_t x = xLane - int32_t(shift); // the lane's first output; the others 64 apart
+    const float* win = tile + r * pitch + (kLine - 1) - shift + lane;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t a = 0; a < KH; ++a)
       for (uint32_t b = 0; b < KW; ++b) {
@@ -170,15 +187,13 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
         if constexpr (KH_ != 0) wt = wreg[a * KW_ + b];
         else wt = wlds[a * KW + b];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + j] * wt + acc[j];
+        for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + 64 * j] * wt + acc[j];
       }
     float* const rowOut = p.out + uint64_t(y) * p.OW; // scalar
-    if (x >= 0 && x + 3 < ow) {
-      streamStore(v4f{acc[0], acc[1], acc[2], acc[3]}, reinterpret_cast<v4f*>(rowOut + x));
-    } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        if (x + j >= 0 && x + j < ow) rowOut[x + j] = acc[j];
+    for (int j = 0; j < 4; ++j) {
+      const int32_t xj = x + 64 * j;
+      if (xj >= 0 && xj < ow) streamStore(acc[j], rowOut + xj);
     }
   }
 }
