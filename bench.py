@@ -586,15 +586,25 @@ def bench_graphs():
         graphs.emit(g, h, {})
         for _ in range(5):
             h.run()
+        c0 = h.counters()
         ts = []
         for _ in range(50):
             t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
         c = h.counters()
+        phases = {name: round((getattr(c, "ns_" + name) - getattr(c0, "ns_" + name)) / 50 / 1e3, 1)
+                  for name in ("input_nodes", "allocate_and_lock", "launch", "release", "barrier")}
         out["logreg_forward"] = {
             "workload": "X[256x784] W[784x10]: 4 input nodes, fmatmul_f_f -> fadd -> fsigmoid -> flogloss, "
                         "one barrier per cluster, inputs re-loaded every evaluation as the framework does",
             "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
-            "launches_per_evaluate": 4, "uploads_per_evaluate": int(c.copies_to_device // 55)}
+            "mean_us": round(float(np.mean(ts)) * 1e6, 1),
+            "phase_us": phases,  # host wall time per evaluation, mean of the 50: the input nodes' host-side
+                                 # loads; per compute node allocate + lock (uploads happen here), the
+                                 # launch call, the releases; the barriers after the clusters
+            "launches_per_evaluate": 4,
+            "uploads_per_evaluate": int((c.copies_to_device - c0.copies_to_device) // 50),
+            "upload_bytes_per_evaluate": int((c.bytes_to_device - c0.bytes_to_device) // 50)}
+        log(f"  phases (us): {phases}")
         log(f"logreg forward through the plugin: {out['logreg_forward']['evaluate_us']} us per evaluation")
     # the same forward pass with the extended (fused) builtins: 2 launches instead of 4
     with harness.Harness(plugin=LIB_PLUGIN) as h:

@@ -45,6 +45,11 @@ typedef struct polar_harness_counters {
   uint64_t deferred_releases; /* releases that ran from event callbacks */
   uint64_t device_name_calls; /* Device::getDeviceName calls on the device
                                  under test (string work the caller causes) */
+  /* host wall time of polar_harness_run by phase, nanoseconds, accumulated:
+   * input nodes (allocate, lock, load, release in host RAM); per compute node
+   * the allocate + lock calls (uploads happen here), the launch call, the
+   * release calls; and the barriers that follow the clusters */
+  uint64_t ns_input_nodes, ns_allocate_and_lock, ns_launch, ns_release, ns_barrier;
 } polar_harness_counters;
 
 /* plugin_path: a runtime plugin to dlopen, or NULL for the built-in CPU mock

@@ -119,8 +119,11 @@ int polar_hip_event_elapsed_ms(polar_hip_event* start, polar_hip_event* stop,
 /* Profiling aid with no counterpart in the reference: the next kernel that an
  * entry point below launches on `dev` carries *start and *stop as its own
  * begin and end timestamps, so polar_hip_event_elapsed_ms(*start, *stop) is
- * that kernel's execution time without launch or queue gaps.  Synchronize
- * *stop before reading; release both events afterwards. */
+ * that kernel's execution time without launch or queue gaps.  Exactly ONE
+ * launch is timed: an entry point that runs several kernels (fsoftmax, a
+ * matmul that splits the contraction) has only its first one bracketed --
+ * time such a call with polar_hip_event_record before and after it instead.
+ * Synchronize *stop before reading; release both events afterwards. */
 int polar_hip_time_next_kernel(polar_hip_device* dev, polar_hip_event** start,
                                polar_hip_event** stop);
 int polar_hip_event_release(polar_hip_event* evt);

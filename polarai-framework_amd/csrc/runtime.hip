@@ -6,6 +6,8 @@
 #include <cstdio>
 #include <cstring>
 
+#include <immintrin.h>
+
 namespace {
 thread_local char g_lastError[512] = "";
 
@@ -297,6 +299,41 @@ hipError_t acquireSlot(polar_hip_device* dev, int* slot) {
 char* slotMemory(polar_hip_device* dev, int slot) {
   return static_cast<char*>(dev->staging) + uint64_t(slot) * kSlotBytes;
 }
+
+// Host copy out of a staging slot into the caller's memory with streaming
+// stores: the destination is written once and not read back by this code, and
+// a regular store would first fetch every destination line into the cache
+// (twice the memory traffic; the C library's memcpy only switches to streaming
+// stores for copies much larger than a slot).
+__attribute__((target("avx2"))) void streamCopyAvx2(char* dst, const char* src, size_t n) {
+  size_t head = (32 - (reinterpret_cast<uintptr_t>(dst) & 31)) & 31;
+  if (head > n) head = n;
+  memcpy(dst, src, head);
+  dst += head;
+  src += head;
+  n -= head;
+  const size_t body = n & ~size_t(127);
+  for (size_t i = 0; i < body; i += 128) {
+    const __m256i a = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(src + i));
+    const __m256i b = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(src + i + 32));
+    const __m256i c = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(src + i + 64));
+    const __m256i d = _mm256_loadu_si256(reinterpret_cast<const __m256i*>(src + i + 96));
+    _mm256_stream_si256(reinterpret_cast<__m256i*>(dst + i), a);
+    _mm256_stream_si256(reinterpret_cast<__m256i*>(dst + i + 32), b);
+    _mm256_stream_si256(reinterpret_cast<__m256i*>(dst + i + 64), c);
+    _mm256_stream_si256(reinterpret_cast<__m256i*>(dst + i + 96), d);
+  }
+  _mm_sfence();
+  memcpy(dst + body, src + body, n - body);
+}
+
+void copyOutOfSlot(void* dst, const void* src, size_t n) {
+  static const bool avx2 = __builtin_cpu_supports("avx2");
+  if (avx2 && n >= (64u << 10))
+    streamCopyAvx2(static_cast<char*>(dst), static_cast<const char*>(src), n);
+  else
+    memcpy(dst, src, n);
+}
 } // namespace
 
 int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
@@ -338,8 +375,7 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
   {
     // Any size: at most kSlots chunk DMAs are in flight; a chunk is copied out
     // as soon as its event completes and its slot goes to the chunk kSlots
-    // further on (256 MiB: 20+ GB/s against 17.6 GB/s for the driver's pageable
-    // path).
+    // further on.
     std::lock_guard<std::mutex> g(dev->stagingMu);
     if (stagingReady(dev)) {
       int slots[kSlots];
@@ -351,7 +387,7 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
         hipError_t e = hipEventSynchronize(dev->slotEvent[slot]);
         if (e != hipSuccess) return e;
         dev->slotBusy[slot] = false;
-        memcpy(static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
+        copyOutOfSlot(static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
         return hipSuccess;
       };
       for (uint64_t c = 0; c < chunks; ++c) {

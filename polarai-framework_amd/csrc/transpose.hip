@@ -15,20 +15,29 @@
 //  * Because b_j differs from row to row, the output rows of a work-group need
 //    input rows from a window that is up to 63 rows tall.  The group therefore
 //    walks down a strip of the input, 32 rows per step, keeping the last two
-//    32 x 256 tiles in an LDS ring; step m emits, for every output row, the
+//    32 x 128 tiles in an LDS ring; step m emits, for every output row, the
 //    aligned chunk that ends inside tile m.  Each input element is read once
 //    per strip (plus one extra tile at the strip's end).
 //  * Input row segments are not line-aligned either, so neighbouring column
-//    tiles share cache lines.  Column tiles are 256 wide (1 KiB segments: two
-//    shared lines per nine) and work-groups are numbered so that each XCD owns
+//    tiles share cache lines.  Work-groups are numbered so that each XCD owns
 //    a contiguous range of column tiles and walks them together: the shared
 //    lines then mostly hit in that XCD's L2 instead of being fetched twice.
 //    For the same reason the loads are plain, not non-temporal (4.7 -> 5.1
 //    TB/s); the stores, which never share a line, stay non-temporal.
-//  * 1024 lanes per group (16 waves): 8 loads per lane in flight, and 32 output
-//    rows per wave in the store phase, two per wave-wide store.
+//  * Shape, measured with rotated buffers on 12345 x 6789 (and seven other
+//    shapes from 333 x 777 to 16384^2): column tiles of 128 with 512 lanes and
+//    strips of 64 rows, 128-130 us; 256 columns with 1024 lanes and strips of
+//    512 rows (fewer, longer-lived groups), 134 us, and 114 instead of 78 us on
+//    50000 x 1000; strips of 32 rows 151 us (every tile is then read twice);
+//    numbering the groups strips-first instead of column-tiles-first 131-138
+//    us.  Only 16384^2 prefers the long strips (445 against 482 us).  The
+//    strip's last tile is read by the next strip as well; that second read
+//    is served by the L2 both groups share.
+//  * 512 lanes per group (8 waves): 8 loads per lane in flight, and 16 output
+//    rows per wave in the store phase, two per wave-wide store.  The ring is
+//    33 KB, so four groups share a CU.
 //
-// The LDS ring has a row pitch of 257 words, so both the row-wise stores of the
+// The LDS ring has a row pitch of 129 words, so both the row-wise stores of the
 // load phase and the column-wise loads of the store phase are conflict-free
 // within a half-wave.  All edges are predicated; any rows x cols works.
 #include "internal.h"
@@ -38,8 +47,8 @@ using namespace polar_hip_detail;
 namespace {
 
 constexpr int kTI = 32;   // input rows per step = elements per aligned output chunk
-constexpr int kTJ = 256;  // input columns (= output rows) per work-group
-constexpr int kThreads = 1024;
+constexpr int kTJ = 128;  // input columns (= output rows) per work-group
+constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / 64;
 constexpr int kLoads = kTI * kTJ / kThreads;    // 8 loads per lane per tile
 constexpr int kColsPerStore = 64 / kTI;         // 2 output rows per wave-wide store
@@ -141,9 +150,9 @@ extern "C" int polar_hip_ftranspose(polar_hip_device* dev, const float* in,
   p.cols = static_cast<uint32_t>(cols);
   p.colTiles = (p.cols + kTJ - 1) / kTJ;
   p.colTilesPerXcd = (p.colTiles + kXcds - 1) / kXcds;
-  // Longest strip (fewest re-read tiles) that still gives every CU two groups.
+  // Strips of 64 rows, shorter when that is needed to give every CU two groups.
   const uint64_t wanted = 2ull * static_cast<uint64_t>(dev->info.compute_units);
-  uint32_t stripRows = 512;
+  uint32_t stripRows = 64;
   while (stripRows > kTI &&
          uint64_t(p.colTiles) * ((p.rows + stripRows - 1) / stripRows) < wanted)
     stripRows /= 2;

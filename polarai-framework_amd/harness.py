@@ -24,7 +24,8 @@ class Arg(C.Structure):
 class Counters(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "launches", "copies_to_device", "bytes_to_device", "copies_to_host",
-        "bytes_to_host", "events_waited", "deferred_releases", "device_name_calls")]
+        "bytes_to_host", "events_waited", "deferred_releases", "device_name_calls",
+        "ns_input_nodes", "ns_allocate_and_lock", "ns_launch", "ns_release", "ns_barrier")]
 
 
 _vp, _u64, _i = C.c_void_p, C.c_uint64, C.c_int

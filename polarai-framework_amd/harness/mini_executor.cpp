@@ -7,6 +7,7 @@
 #include <dlfcn.h>
 
 #include <cstdio>
+#include <chrono>
 #include <cstring>
 
 using namespace polar_harness_detail;
@@ -282,18 +283,26 @@ int polar_harness_run(polar_harness* h) {
       }
 
   const uint64_t deferred0 = g_deferredReleases, waited0 = g_eventsWaited;
+  using Clock = std::chrono::steady_clock;
+  auto since = [](Clock::time_point t0) {
+    return static_cast<uint64_t>(
+        std::chrono::duration_cast<std::chrono::nanoseconds>(Clock::now() - t0).count());
+  };
   for (auto& cluster : h->clusters) {
     std::vector<Event*> events;
     for (auto& n : cluster) {
       Device* dev = ath_device_select(&gh, n.id);
       if (n.isInput) {
+        const auto t0 = Clock::now();
         TensorInfo ti = h->find(n.inputVaddr)->info();
         ath_allocate(&gh, *dev, &ti);
         ath_lock(&gh, *dev, &ti, LockType::READ_WRITE);
         ath_load(&gh, n.id, &ti);
         ath_release(&gh, *dev, &ti, nullptr);
+        h->counters.ns_input_nodes += since(t0);
         continue;
       }
+      auto t0 = Clock::now();
       std::vector<TensorInfo> infos(n.args.size());
       std::vector<ArgDesc> descs(n.args.size());
       std::vector<float> scalars(n.args.size());
@@ -325,12 +334,21 @@ int polar_harness_run(polar_harness* h) {
       const std::string jitName =
           n.jitName.empty() ? "node" + std::to_string(n.id) + "_" + n.kernel : n.jitName;
       LaunchCommand cmd{jitName.c_str(), descs.size(), descs.data(), n.kernel.c_str()};
+      h->counters.ns_allocate_and_lock += since(t0);
+      t0 = Clock::now();
       Event* evt = ath_launch(&gh, dev, nullptr, cmd);
+      h->counters.ns_launch += since(t0);
+      t0 = Clock::now();
       for (size_t i : readLocked) ath_release(&gh, *dev, &infos[i], evt);
       ath_release(&gh, *dev, &infos[n.result], evt);
       events.push_back(evt);
+      h->counters.ns_release += since(t0);
     }
-    if (!events.empty()) ath_barrier(static_cast<uint32_t>(events.size()), events.data());
+    if (!events.empty()) {
+      const auto t0 = Clock::now();
+      ath_barrier(static_cast<uint32_t>(events.size()), events.data());
+      h->counters.ns_barrier += since(t0);
+    }
   }
   h->counters.deferred_releases += g_deferredReleases - deferred0;
   h->counters.events_waited += g_eventsWaited - waited0;

@@ -153,16 +153,19 @@ bool HipDevice::launchFromProgram(BackendAllocator& allocator, LaunchCommand& cm
   std::vector<int64_t> integers;        // offsets, sizes, strides
   std::vector<std::pair<int, size_t>> layout; // (0 pointer / 1 integer / 2 scalar, index)
   uint64_t tensors = 0, words = 0;
-  for (uint64_t i = 0; i < cmd.argsCount; ++i)
+  for (uint64_t i = 0; i < cmd.argsCount; ++i) {
+    // validated before the first use: the sizing pass below reads the tensor's rank
+    if (cmd.args[i].arg == nullptr)
+      fatal("%s: argument %llu is null", cmd.kernelName, (unsigned long long)i);
     if (cmd.args[i].type == ArgDesc::TENSOR) {
       ++tensors;
       words += 1 + 2 * static_cast<TensorInfo*>(cmd.args[i].arg)->dims;
     }
+  }
   pointers.reserve(2 * tensors); // addresses of the elements are taken below
   integers.reserve(words);
   for (uint64_t i = 0; i < cmd.argsCount; ++i) {
     const ArgDesc& a = cmd.args[i];
-    if (a.arg == nullptr) fatal("%s: argument %llu is null", cmd.kernelName, (unsigned long long)i);
     if (a.type != ArgDesc::TENSOR) {
       layout.emplace_back(2, i);
       continue;
