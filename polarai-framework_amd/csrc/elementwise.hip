@@ -308,18 +308,18 @@ static_assert(kSumRounds * kSumBatch * kSumBlock * 4 == kSumChunk, "chunk is who
 // exp(x) for the terms of the sum: 2^n * 2^r with n = round(x log2 e) and
 // r = x log2 e - n in [-0.5, 0.5] computed with two fused multiply-adds (log2 e
 // split into a high and a low part), the hardware's exp2 for 2^r and ldexp for
-// the scaling, which also produces the overflow to infinity and the underflow
-// to zero.  7 instructions instead of the 13 of the library's expf (which
-// spends the difference on range checks that the clamp below replaces); with
-// them the pass was bound by instruction issue, not by memory.  The error is
-// below 1.5 units in the last place; the total only enters the result through
-// its fp32 rounding.  NaN stays NaN; the clamp keeps x log2 e inside the
-// integer range (exp overflows above 88.73 and is 0 below -103.98 anyway).
+// the scaling.  8 instructions instead of the 13 of the library's expf (which
+// spends the difference on range checks); with those the pass was bound by
+// instruction issue, not by memory.  The error is below 1.5 units in the last
+// place; the total only enters the result through its fp32 rounding.
+// Only n is computed from a clamped argument (so that it fits an integer; exp
+// overflows above 88.73 and is 0 below -103.98 anyway); r uses x itself, so
+// beyond the clamp r is huge and exp2 returns the infinity or the zero that is
+// due, +-infinity included, and a NaN stays a NaN.
 __device__ __forceinline__ float expTerm(float x) {
   const float kLog2eHi = 1.44269502162933349609375f; // fp32 nearest to log2 e
   const float kLog2eLo = 1.925963033500011e-8f;      // log2 e - kLog2eHi
-  x = __builtin_amdgcn_fmed3f(x, -104.0f, 89.0f);
-  const float n = __builtin_rintf(x * kLog2eHi);
+  const float n = __builtin_rintf(__builtin_amdgcn_fmed3f(x, -104.0f, 89.0f) * kLog2eHi);
   float r = __builtin_fmaf(x, kLog2eHi, -n);
   r = __builtin_fmaf(x, kLog2eLo, r);
   return __builtin_amdgcn_ldexpf(__builtin_amdgcn_exp2f(r), static_cast<int>(n));

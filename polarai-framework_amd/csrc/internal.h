@@ -53,15 +53,12 @@ struct polar_hip_device {
   void* softmaxScratch = nullptr;
 
   // Workspace of the builtins that run more than one kernel per call (softmax
-  // partial sums, split-K partial products).  Allocated when the device is
-  // opened, so a launch neither allocates nor waits; a call that needs more
-  // replaces it by one twice as large, and the outgrown block stays until the
-  // device is closed because kernels already enqueued may still use it.
-  // workspaceMu is held while a call enqueues the kernels that share it.
+  // partial sums, split-K partial products): one block allocated when the
+  // device is opened and sized for the largest request the library makes, so
+  // that a launch neither allocates nor waits.  workspaceMu is held while a
+  // call enqueues the kernels that share it.
   std::mutex workspaceMu;
   void* workspace = nullptr;
-  uint64_t workspaceBytes = 0;
-  std::vector<void*> outgrownWorkspaces;
 };
 
 struct polar_hip_module {
@@ -79,10 +76,11 @@ int fail(polar_hip_status st, const char* fmt, ...)
 int failHip(hipError_t e, const char* what);
 int resolveStaticScratch(polar_hip_device* dev); // elementwise.hip
 
-constexpr uint64_t kInitialWorkspace = 64ull << 20;
-// *area: at least `bytes` of device memory, 256-byte aligned, contents
-// undefined.  Caller holds dev->workspaceMu.  Allocates only when `bytes`
-// exceeds what the device holds.
+// The matmul planner never asks for more split-K workspace than this, and the
+// partial sums of a softmax over 2^31 elements take 256 KiB.
+constexpr uint64_t kWorkspaceBytes = 256ull << 20;
+// *area: the device's workspace (kWorkspaceBytes, 256-byte aligned, contents
+// undefined).  Caller holds dev->workspaceMu.  Fails for a larger request.
 int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area); // runtime.hip
 
 // Every kernel of the library is launched through here.  Normally a plain

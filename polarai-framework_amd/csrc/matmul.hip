@@ -440,7 +440,7 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
     const uint32_t kSteps = (k + t.bk - 1) / t.bk;
     const double mfmaUs = 2.0 * t.bm * t.bn * t.bk / (256.0 * 2400.0 * t.mfmaEfficiency);
     for (uint32_t s : kSplitChoices) {
-      if (s > 1 && (kSteps / s < 2 || double(m) * n * s * 4 > double(256u << 20))) break;
+      if (s > 1 && (kSteps / s < 2 || double(m) * n * s * 4 > double(kWorkspaceBytes))) break;
       const double groups = tiles * s;
       double resident = groups / computeUnits;
       if (resident < 1) resident = 1;

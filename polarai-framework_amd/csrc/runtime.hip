@@ -44,16 +44,9 @@ int failHip(hipError_t e, const char* what) {
 // ---- workspace ----------------------------------------------------------------
 
 int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area) {
-  if (bytes > dev->workspaceBytes) {
-    uint64_t wanted = dev->workspaceBytes ? dev->workspaceBytes : kInitialWorkspace;
-    while (wanted < bytes) wanted *= 2;
-    POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-    void* block = nullptr;
-    POLAR_HIP_TRY(hipMalloc(&block, wanted));
-    if (dev->workspace) dev->outgrownWorkspaces.push_back(dev->workspace);
-    dev->workspace = block;
-    dev->workspaceBytes = wanted;
-  }
+  if (bytes > kWorkspaceBytes)
+    return fail(POLAR_HIP_ERR_INVALID, "workspace request of %llu bytes exceeds the %llu the device holds",
+                static_cast<unsigned long long>(bytes), static_cast<unsigned long long>(kWorkspaceBytes));
   *area = dev->workspace;
   return POLAR_HIP_OK;
 }
@@ -116,9 +109,8 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
   d->info.hbm_bytes = p.totalGlobalMem;
   st = resolveStaticScratch(d);
   if (st == POLAR_HIP_OK) {
-    std::lock_guard<std::mutex> g(d->workspaceMu);
-    void* unused = nullptr;
-    st = polar_hip_detail::workspaceFor(d, polar_hip_detail::kInitialWorkspace, &unused);
+    e = hipMalloc(&d->workspace, polar_hip_detail::kWorkspaceBytes);
+    if (e != hipSuccess) st = failHip(e, "hipMalloc (workspace)");
   }
   if (st != POLAR_HIP_OK) {
     (void)hipStreamDestroy(d->stream);
@@ -137,7 +129,6 @@ int polar_hip_device_close(polar_hip_device* dev) {
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : dev->live) (void)hipFree(kv.first);
   if (dev->workspace) (void)hipFree(dev->workspace);
-  for (void* p : dev->outgrownWorkspaces) (void)hipFree(p);
   for (auto* e : dev->allEvents) {
     (void)hipEventDestroy(e->ev);
     delete e;

@@ -319,6 +319,49 @@ def test_transpose_matmul_cross_identity(dev):
         x.free()
 
 
+def test_split_contraction_and_softmax_allocate_nothing(dev):
+    """Calls that run more than one kernel (a matmul that splits the
+    contraction, fsoftmax) work in the block the device holds since it was
+    opened: the pool's counters do not move, first call included."""
+    rng = np.random.default_rng(51)
+    m, n, k = 300, 260, 40000      # 4 tiles of 256 x 256 at most: the contraction is split
+    a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+    b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+    da, db, dc = dev.array(a), dev.array(b), dev.empty(m * n)
+    dx, dy = dev.array(parity.normal(rng, 300000)), dev.empty(300000)
+    dev.synchronize()
+    s0 = dev.pool_stats()
+    for _ in range(2):
+        dev.fmatmul(False, False, da, db, dc, m, n, k)
+        dev.fsoftmax(dx, dy)
+    s1 = dev.pool_stats()
+    assert (s1.device_allocs, s1.pool_hits, s1.bytes_in_use, s1.bytes_cached) == \
+           (s0.device_allocs, s0.pool_hits, s0.bytes_in_use, s0.bytes_cached)
+    ref = a.astype(np.float64) @ b.astype(np.float64)     # integers: exact in fp32
+    assert np.array_equal(dc.download((m, n)), ref.astype(np.float32))
+    for t in (da, db, dc, dx, dy):
+        t.free()
+
+
+@pytest.mark.parametrize("nbytes", [65536, 65536 + 4, 512 * 1024 + 12, 3 * 1024 * 1024 + 100])
+@pytest.mark.parametrize("offset", [0, 4, 36])
+def test_copy_to_host_into_unaligned_memory(dev, nbytes, offset):
+    """Large read-backs are drained from the staging ring with streaming stores
+    (aligned body, ordinary head and tail): every byte must arrive, and nothing
+    outside the destination may change."""
+    _say("copy_to_host", nbytes, offset)
+    count = nbytes // 4
+    src = np.arange(count, dtype=np.float32)
+    d = dev.array(src)
+    guard = 64
+    raw = np.full(nbytes + offset + 2 * guard, 0x5A, dtype=np.uint8)
+    dst = raw[guard + offset: guard + offset + nbytes]
+    dev.copy_to_host(dst.ctypes.data, d.ptr, nbytes)
+    assert np.array_equal(dst.view(np.float32) if offset % 4 == 0 else np.frombuffer(dst.tobytes(), np.float32), src)
+    assert np.all(raw[:guard + offset] == 0x5A) and np.all(raw[guard + offset + nbytes:] == 0x5A)
+    d.free()
+
+
 def test_pool_reuses_blocks(dev):
     dev.synchronize()
     s0 = dev.pool_stats()
@@ -373,6 +416,52 @@ def test_softmax_against_sequential_oracle(dev, n):
         assert parity.elementwise_rel_error(got, o.fsoftmax(x)) <= parity.ELEMENTWISE_REL
         assert parity.elementwise_rel_error(got, o.fsoftmax(x, f64sum=True)) <= 2e-6
         dx.free(); dout.free()
+
+
+def test_softmax_sum_over_the_exponent_range(dev):
+    """The sum pass has an exponential of its own: checked where that could
+    differ from the library's -- arguments from deep underflow to just below
+    overflow, with the total dominated by few large terms and by many small
+    ones -- against the fp64-accumulated oracle."""
+    rng = np.random.default_rng(811)
+    n = 70001   # one full vector chunk and a ragged tail
+    cases = {
+        "wide": rng.uniform(-100.0, 80.0, n).astype(np.float32),
+        "negative": rng.uniform(-103.0, -60.0, n).astype(np.float32),
+        "near overflow": rng.uniform(70.0, 87.0, n).astype(np.float32),
+        "small": (rng.standard_normal(n) * 1e-3).astype(np.float32),
+    }
+    cases["wide"][:5] = [0.0, -103.5, -104.5, 79.99, -0.0]
+    for label, x in cases.items():
+        _say("softmax range", label)
+        dx, dout = dev.array(x), dev.empty(n)
+        dev.fsoftmax(dx, dout)
+        got = dout.download()
+        ref = o.fsoftmax(x, f64sum=True)
+        assert np.all(np.isfinite(got)), label
+        assert parity.elementwise_rel_error(got, ref) <= 2e-6, label
+        dx.free(); dout.free()
+
+
+@pytest.mark.parametrize("special", [89.0, np.inf, np.nan, -np.inf])
+def test_softmax_special_values_follow_the_reference(dev, special):
+    """An argument whose exponential overflows makes the total infinite (finite
+    terms become 0, the overflowing one inf/inf = NaN); a NaN makes everything
+    NaN; -inf contributes 0.  Same pattern as the oracle's loop."""
+    _say("softmax special", special)
+    n = 65536 + 17
+    x = parity.normal(np.random.default_rng(812), n)
+    x[n // 2] = special
+    x[n - 3] = special
+    dx, dout = dev.array(x), dev.empty(n)
+    dev.fsoftmax(dx, dout)
+    got = dout.download()
+    with np.errstate(all="ignore"):
+        ref = o.fsoftmax(x, f64sum=True)
+    assert np.array_equal(np.isnan(got), np.isnan(ref))
+    keep = ~np.isnan(ref)
+    assert parity.elementwise_rel_error(got[keep], ref[keep]) <= 2e-6
+    dx.free(); dout.free()
 
 
 def test_softmax_is_repeatable(dev):

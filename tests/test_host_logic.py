@@ -29,6 +29,13 @@ def test_device_library_exports_every_declared_symbol():
     assert sorted(capi.SIGNATURES) == names  # the binding covers the header exactly
 
 
+def test_probe_library_exports_what_the_benchmark_calls():
+    from polarai_framework_amd import LIB_PROBES
+    lib = C.CDLL(LIB_PROBES)
+    for name in ("polar_probe_streams", "polar_probe_read", "polar_probe_transpose_pattern"):
+        assert hasattr(lib, name), name
+
+
 def test_harness_library_exports_every_declared_symbol():
     names = _declared("polar_harness.h", "polar_harness_")
     lib = C.CDLL(LIB_HARNESS)
