@@ -7,11 +7,13 @@
 #include <hip/hip_ext.h>
 
 #include <cstdarg>
+#include <condition_variable>
 #include <cstdint>
 #include <map>
 #include <memory>
 #include <mutex>
 #include <string>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -20,6 +22,22 @@
 struct polar_hip_event {
   polar_hip_device* dev;
   hipEvent_t ev;
+};
+
+// Second host thread of large device-to-host copies: the staging slots are
+// drained into the caller's memory by two threads, because one thread's copy
+// rate (about 22 GB/s) is below what the DMA engine delivers.  It takes one job
+// at a time; started on the first copy that uses it, joined when the device is
+// closed.
+struct DrainThread {
+  std::thread thread;
+  std::mutex mu;
+  std::condition_variable cv;
+  char* dst = nullptr;
+  const char* src = nullptr;
+  size_t bytes = 0;
+  bool pending = false; // a job is posted and not yet finished
+  bool quit = false;
 };
 
 struct polar_hip_device {
@@ -42,6 +60,7 @@ struct polar_hip_device {
   hipEvent_t slotEvent[8] = {};
   bool slotBusy[8] = {};
   int nextSlot = 0;
+  DrainThread drain; // used under stagingMu
 
   // armed by polar_hip_time_next_kernel: the next kernel launch carries these
   // as its start/stop events

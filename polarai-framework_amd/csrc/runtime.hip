@@ -10,6 +10,7 @@
 
 namespace {
 thread_local char g_lastError[512] = "";
+void drainStop(DrainThread& d); // with the copy code below
 
 uint64_t roundBlock(uint64_t bytes) {
   // Small blocks: powers of two from 256 B.  Large blocks: multiples of 2 MiB,
@@ -133,6 +134,7 @@ int polar_hip_device_close(polar_hip_device* dev) {
     (void)hipEventDestroy(e->ev);
     delete e;
   }
+  drainStop(dev->drain);
   if (dev->staging) {
     for (hipEvent_t e : dev->slotEvent) (void)hipEventDestroy(e);
     (void)hipHostFree(dev->staging);
@@ -236,28 +238,33 @@ int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out) {
 
 // ---- copies -----------------------------------------------------------------
 // Host memory handed in by the framework is pageable.  The driver's pageable
-// path is fast for large transfers (30 GB/s up, 18 GB/s down, measured) but has
-// a high fixed cost for small and medium ones (110 us for 256 KiB), which is
-// what graph inputs and read-backs mostly are.  Uploads of up to 4 MiB and all
-// downloads go through a ring of pinned 512 KiB slots instead:
+// path has a high fixed cost for small and medium transfers (110 us for 256
+// KiB), which is what graph inputs and read-backs mostly are, and reaches 30
+// GB/s up and 18 GB/s down on large ones.  All copies go through a ring of
+// eight pinned slots instead:
 //  * upload: the source is copied into a slot and the DMA is enqueued on the
 //    device's stream; the call returns without waiting for it (the caller's
 //    buffer is already free, and everything that uses the destination is
 //    ordered after the DMA on the same stream).  A slot is reused only after
 //    the event recorded behind its DMA has completed.
-//  * download: up to eight chunk DMAs are kept in flight and each chunk is
-//    copied out as soon as its event completes, so the host copy of one chunk
-//    overlaps the DMA of the next ones.
+//  * download: chunk DMAs are kept in flight and each chunk is copied out as
+//    soon as its event completes, so the host copy of one chunk overlaps the
+//    DMA of the next ones.
+//  * transfers below 8 MiB move in 512 KiB chunks (the first DMA starts early);
+//    larger ones in 2 MiB chunks (about 10 us of driver calls per chunk
+//    otherwise cap the rate) with a second host thread taking every second
+//    chunk's host-side copy: 256 MiB read back at 40 GB/s instead of 22.
 namespace {
-constexpr uint64_t kSlotBytes = 512ull << 10;
+constexpr uint64_t kSlotBytes = 512ull << 10;     // chunk of uploads and of small and medium read-backs
+constexpr uint64_t kSlotCapacity = 2ull << 20;    // a slot's memory; large read-backs use all of it
 constexpr int kSlots = 8;
-constexpr uint64_t kStagingBytes = kSlotBytes * kSlots;
+constexpr uint64_t kTwoThreadBytes = 8ull << 20;  // copies from this size on use whole slots and the drain thread
 
 // called with dev->stagingMu held
 bool stagingReady(polar_hip_device* dev) {
   if (dev->staging != nullptr) return true;
   void* p = nullptr;
-  if (hipHostMalloc(&p, kStagingBytes, hipHostMallocDefault) != hipSuccess) {
+  if (hipHostMalloc(&p, kSlotCapacity * kSlots, hipHostMallocDefault) != hipSuccess) {
     (void)hipGetLastError();
     return false;
   }
@@ -288,11 +295,11 @@ hipError_t acquireSlot(polar_hip_device* dev, int* slot) {
 }
 
 char* slotMemory(polar_hip_device* dev, int slot) {
-  return static_cast<char*>(dev->staging) + uint64_t(slot) * kSlotBytes;
+  return static_cast<char*>(dev->staging) + uint64_t(slot) * kSlotCapacity;
 }
 
-// Host copy out of a staging slot into the caller's memory with streaming
-// stores: the destination is written once and not read back by this code, and
+// Host copy between a staging slot and the caller's memory with streaming
+// stores: the destination is written once and not read back by this thread, and
 // a regular store would first fetch every destination line into the cache
 // (twice the memory traffic; the C library's memcpy only switches to streaming
 // stores for copies much larger than a slot).
@@ -318,6 +325,48 @@ __attribute__((target("avx2"))) void streamCopyAvx2(char* dst, const char* src, 
   memcpy(dst + body, src + body, n - body);
 }
 
+void copyOutOfSlot(void* dst, const void* src, size_t n);
+
+void drainLoop(DrainThread* d) {
+  std::unique_lock<std::mutex> lock(d->mu);
+  for (;;) {
+    d->cv.wait(lock, [&] { return d->pending || d->quit; });
+    if (d->quit) return;
+    char* dst = d->dst;
+    const char* src = d->src;
+    const size_t n = d->bytes;
+    lock.unlock();
+    copyOutOfSlot(dst, src, n);
+    lock.lock();
+    d->pending = false;
+    d->cv.notify_all();
+  }
+}
+// wait until the drain thread has finished the job it holds, if any
+void drainWait(DrainThread& d) {
+  std::unique_lock<std::mutex> lock(d.mu);
+  d.cv.wait(lock, [&] { return !d.pending; });
+}
+void drainPost(DrainThread& d, char* dst, const char* src, size_t n) {
+  std::unique_lock<std::mutex> lock(d.mu);
+  d.cv.wait(lock, [&] { return !d.pending; });
+  if (!d.thread.joinable()) d.thread = std::thread(drainLoop, &d);
+  d.dst = dst;
+  d.src = src;
+  d.bytes = n;
+  d.pending = true;
+  d.cv.notify_all();
+}
+void drainStop(DrainThread& d) {
+  {
+    std::unique_lock<std::mutex> lock(d.mu);
+    d.cv.wait(lock, [&] { return !d.pending; });
+    d.quit = true;
+    d.cv.notify_all();
+  }
+  if (d.thread.joinable()) d.thread.join();
+}
+
 void copyOutOfSlot(void* dst, const void* src, size_t n) {
   static const bool avx2 = __builtin_cpu_supports("avx2");
   if (avx2 && n >= (64u << 10))
@@ -334,19 +383,52 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
   POLAR_HIP_REQUIRE(dst_device != nullptr && src_host != nullptr,
                     "null buffer");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-  if (bytes <= kStagingBytes) {
+  {
+    // The data is copied into pinned slots and sent from there, so the call
+    // returns once the last DMA is queued and the caller may reuse its memory.
+    // From kTwoThreadBytes on, slots are filled whole (2 MiB) and every second
+    // one by the drain thread: one thread fills at about 30 GB/s, less than
+    // the link takes.
     std::lock_guard<std::mutex> g(dev->stagingMu);
     if (stagingReady(dev)) {
-      for (uint64_t off = 0; off < bytes; off += kSlotBytes) {
-        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
-        int slot;
-        POLAR_HIP_TRY(acquireSlot(dev, &slot));
-        memcpy(slotMemory(dev, slot), static_cast<const char*>(src_host) + off, n);
-        POLAR_HIP_TRY(hipMemcpyAsync(static_cast<char*>(dst_device) + off, slotMemory(dev, slot),
-                                     n, hipMemcpyHostToDevice, dev->stream));
-        POLAR_HIP_TRY(hipEventRecord(dev->slotEvent[slot], dev->stream));
-        dev->slotBusy[slot] = true;
+      const bool twoThreads = bytes >= kTwoThreadBytes;
+      const uint64_t chunkBytes = twoThreads ? kSlotCapacity : kSlotBytes;
+      const char* src = static_cast<const char*>(src_host);
+      char* dst = static_cast<char*>(dst_device);
+      auto send = [&](int slot, uint64_t off, uint64_t n) -> hipError_t {
+        hipError_t e = hipMemcpyAsync(dst + off, slotMemory(dev, slot), n, hipMemcpyHostToDevice, dev->stream);
+        if (e != hipSuccess) return e;
+        e = hipEventRecord(dev->slotEvent[slot], dev->stream);
+        if (e == hipSuccess) dev->slotBusy[slot] = true;
+        return e;
+      };
+      hipError_t failed = hipSuccess;
+      for (uint64_t off = 0; off < bytes && failed == hipSuccess; off += 2 * chunkBytes) {
+        const uint64_t nA = bytes - off < chunkBytes ? bytes - off : chunkBytes;
+        const uint64_t offB = off + nA;
+        const uint64_t nB = bytes - offB < chunkBytes ? bytes - offB : chunkBytes;
+        int slotA, slotB = -1;
+        failed = acquireSlot(dev, &slotA);
+        if (failed != hipSuccess) break;
+        if (twoThreads && nB > 0) {
+          failed = acquireSlot(dev, &slotB);
+          if (failed != hipSuccess) break;
+          drainPost(dev->drain, slotMemory(dev, slotB), src + offB, nB);
+        }
+        if (twoThreads) copyOutOfSlot(slotMemory(dev, slotA), src + off, nA);
+        else memcpy(slotMemory(dev, slotA), src + off, nA);
+        failed = send(slotA, off, nA);
+        if (slotB >= 0) {
+          drainWait(dev->drain); // even if the send failed: the thread holds a job
+          if (failed == hipSuccess) failed = send(slotB, offB, nB);
+        } else if (failed == hipSuccess && nB > 0) {
+          failed = acquireSlot(dev, &slotB);
+          if (failed != hipSuccess) break;
+          memcpy(slotMemory(dev, slotB), src + offB, nB);
+          failed = send(slotB, offB, nB);
+        }
       }
+      if (failed != hipSuccess) return failHip(failed, "host-to-device copy");
       return POLAR_HIP_OK;
     }
   }
@@ -366,36 +448,56 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
   {
     // Any size: at most kSlots chunk DMAs are in flight; a chunk is copied out
     // as soon as its event completes and its slot goes to the chunk kSlots
-    // further on.
+    // further on.  In a large transfer every second chunk is copied out by the
+    // drain thread while this thread goes on to the next one.  The thread holds
+    // one job at a time and posting a job waits for the previous one, so chunks
+    // are consumed kSlots - 2 behind the DMAs instead of kSlots: when chunk i is
+    // about to take the slot of chunk i - kSlots, chunk i - kSlots + 2 (same
+    // parity) has just been posted or copied, which means the copy of chunk
+    // i - kSlots has finished, whichever thread made it.
     std::lock_guard<std::mutex> g(dev->stagingMu);
     if (stagingReady(dev)) {
       int slots[kSlots];
-      const uint64_t chunks = (bytes + kSlotBytes - 1) / kSlotBytes;
+      const bool twoThreads = bytes >= kTwoThreadBytes;
+      // per chunk this thread pays about 10 us of driver calls; with 512 KiB
+      // chunks that alone capped a 256 MiB read-back at 24 GB/s
+      const uint64_t chunkBytes = twoThreads ? kSlotCapacity : kSlotBytes;
+      const uint64_t chunks = (bytes + chunkBytes - 1) / chunkBytes;
       auto consume = [&](uint64_t c) -> hipError_t {
-        const uint64_t off = c * kSlotBytes;
-        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
+        const uint64_t off = c * chunkBytes;
+        const uint64_t n = bytes - off < chunkBytes ? bytes - off : chunkBytes;
         const int slot = slots[c % kSlots];
         hipError_t e = hipEventSynchronize(dev->slotEvent[slot]);
         if (e != hipSuccess) return e;
         dev->slotBusy[slot] = false;
-        copyOutOfSlot(static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
+        if (twoThreads && (c & 1))
+          drainPost(dev->drain, static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
+        else
+          copyOutOfSlot(static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
         return hipSuccess;
       };
-      for (uint64_t c = 0; c < chunks; ++c) {
-        if (c >= kSlots) POLAR_HIP_TRY(consume(c - kSlots));
-        const uint64_t off = c * kSlotBytes;
-        const uint64_t n = bytes - off < kSlotBytes ? bytes - off : kSlotBytes;
+      const uint64_t lag = twoThreads ? kSlots - 2 : kSlots;
+      hipError_t failed = hipSuccess;
+      for (uint64_t c = 0; c < chunks && failed == hipSuccess; ++c) {
+        if (c >= lag) failed = consume(c - lag);
+        if (failed != hipSuccess) break;
+        const uint64_t off = c * chunkBytes;
+        const uint64_t n = bytes - off < chunkBytes ? bytes - off : chunkBytes;
         int slot;
-        POLAR_HIP_TRY(acquireSlot(dev, &slot));
+        failed = acquireSlot(dev, &slot);
+        if (failed != hipSuccess) break;
         slots[c % kSlots] = slot;
-        POLAR_HIP_TRY(hipMemcpyAsync(slotMemory(dev, slot),
-                                     static_cast<const char*>(src_device) + off, n,
-                                     hipMemcpyDeviceToHost, dev->stream));
-        POLAR_HIP_TRY(hipEventRecord(dev->slotEvent[slot], dev->stream));
+        failed = hipMemcpyAsync(slotMemory(dev, slot), static_cast<const char*>(src_device) + off, n,
+                                hipMemcpyDeviceToHost, dev->stream);
+        if (failed != hipSuccess) break;
+        failed = hipEventRecord(dev->slotEvent[slot], dev->stream);
+        if (failed != hipSuccess) break;
         dev->slotBusy[slot] = true;
       }
-      for (uint64_t c = chunks > kSlots ? chunks - kSlots : 0; c < chunks; ++c)
-        POLAR_HIP_TRY(consume(c));
+      for (uint64_t c = chunks > lag ? chunks - lag : 0; c < chunks && failed == hipSuccess; ++c)
+        failed = consume(c);
+      if (twoThreads) drainWait(dev->drain); // also on failure: the thread may still hold a job
+      if (failed != hipSuccess) return failHip(failed, "device-to-host copy");
       return POLAR_HIP_OK;
     }
   }

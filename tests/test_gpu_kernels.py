@@ -343,15 +343,17 @@ def test_split_contraction_and_softmax_allocate_nothing(dev):
         t.free()
 
 
-@pytest.mark.parametrize("nbytes", [65536, 65536 + 4, 512 * 1024 + 12, 3 * 1024 * 1024 + 100])
+@pytest.mark.parametrize("nbytes", [65536, 65536 + 4, 512 * 1024 + 12, 3 * 1024 * 1024 + 100,
+                                    8 * 1024 * 1024, 9 * 1024 * 1024 + 20, 41 * 1024 * 1024 + 4])
 @pytest.mark.parametrize("offset", [0, 4, 36])
 def test_copy_to_host_into_unaligned_memory(dev, nbytes, offset):
     """Large read-backs are drained from the staging ring with streaming stores
-    (aligned body, ordinary head and tail): every byte must arrive, and nothing
+    (aligned body, ordinary head and tail), from 8 MiB on by two host threads
+    that take alternate chunks: every byte must arrive in place, and nothing
     outside the destination may change."""
     _say("copy_to_host", nbytes, offset)
     count = nbytes // 4
-    src = np.arange(count, dtype=np.float32)
+    src = (np.arange(count, dtype=np.int64) % 16000057).astype(np.float32)   # distinct per chunk position
     d = dev.array(src)
     guard = 64
     raw = np.full(nbytes + offset + 2 * guard, 0x5A, dtype=np.uint8)
@@ -359,6 +361,22 @@ def test_copy_to_host_into_unaligned_memory(dev, nbytes, offset):
     dev.copy_to_host(dst.ctypes.data, d.ptr, nbytes)
     assert np.array_equal(dst.view(np.float32) if offset % 4 == 0 else np.frombuffer(dst.tobytes(), np.float32), src)
     assert np.all(raw[:guard + offset] == 0x5A) and np.all(raw[guard + offset + nbytes:] == 0x5A)
+    d.free()
+
+
+@pytest.mark.parametrize("nbytes", [4 * 1024 * 1024 + 8, 8 * 1024 * 1024, 10 * 1024 * 1024 + 4,
+                                    13 * 1024 * 1024 + 36])
+def test_copy_to_device_of_large_buffers_round_trips(dev, nbytes):
+    """Uploads from 8 MiB on fill whole staging slots with two host threads; the
+    source may be reused as soon as the call returns."""
+    _say("copy_to_device", nbytes)
+    count = nbytes // 4
+    src = (np.arange(count, dtype=np.int64) % 16000057).astype(np.float32)
+    keep = src.copy()
+    d = dev.empty(count)
+    dev.copy_to_device(d.ptr, src.ctypes.data, nbytes)
+    src[:] = -1.0                      # the call has taken its copy
+    assert np.array_equal(d.download(), keep)
     d.free()
 
 
