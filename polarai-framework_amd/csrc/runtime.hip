@@ -327,6 +327,24 @@ __attribute__((target("avx2"))) void streamCopyAvx2(char* dst, const char* src, 
 
 void copyOutOfSlot(void* dst, const void* src, size_t n);
 
+// Upload of one staging slot by the compute units instead of the DMA engine:
+// the slot is pinned host memory that the GPU can address, so a kernel on the
+// device's own queue reads it across the link and writes HBM.  Work that
+// follows on the stream then starts as soon as the kernel retires; behind a
+// DMA-engine copy it waits for a signal from another engine, which costs
+// 10-15 us per upload in a graph whose kernels run for 2-10 us.
+typedef float upload_v4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void uploadKernel(const upload_v4* src, upload_v4* dst, uint32_t vectors,
+                                                    uint32_t tailBytes) {
+  const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+  if (i < vectors) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
+  if (blockIdx.x == 0 && threadIdx.x < tailBytes) {
+    const char* s = reinterpret_cast<const char*>(src + vectors);
+    char* d = reinterpret_cast<char*>(dst + vectors);
+    d[threadIdx.x] = s[threadIdx.x];
+  }
+}
+
 void drainLoop(DrainThread* d) {
   std::unique_lock<std::mutex> lock(d->mu);
   for (;;) {
@@ -396,7 +414,16 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
       const char* src = static_cast<const char*>(src_host);
       char* dst = static_cast<char*>(dst_device);
       auto send = [&](int slot, uint64_t off, uint64_t n) -> hipError_t {
-        hipError_t e = hipMemcpyAsync(dst + off, slotMemory(dev, slot), n, hipMemcpyHostToDevice, dev->stream);
+        hipError_t e;
+        if (!twoThreads && (reinterpret_cast<uintptr_t>(dst + off) & 15u) == 0) {
+          const uint32_t vectors = static_cast<uint32_t>(n / 16), tail = static_cast<uint32_t>(n % 16);
+          hipLaunchKernelGGL(uploadKernel, dim3(vectors / 256 + 1), dim3(256), 0, dev->stream,
+                             reinterpret_cast<const upload_v4*>(slotMemory(dev, slot)),
+                             reinterpret_cast<upload_v4*>(dst + off), vectors, tail);
+          e = hipGetLastError();
+        } else {
+          e = hipMemcpyAsync(dst + off, slotMemory(dev, slot), n, hipMemcpyHostToDevice, dev->stream);
+        }
         if (e != hipSuccess) return e;
         e = hipEventRecord(dev->slotEvent[slot], dev->stream);
         if (e == hipSuccess) dev->slotBusy[slot] = true;
@@ -415,6 +442,9 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
           if (failed != hipSuccess) break;
           drainPost(dev->drain, slotMemory(dev, slotB), src + offB, nB);
         }
+        // below the two-thread size a plain memcpy: the source is usually still in
+        // the cache, and the GPU's reads of the slot are served from there too
+        // (streaming stores measured 5 us slower on an 800 KB graph input)
         if (twoThreads) copyOutOfSlot(slotMemory(dev, slotA), src + off, nA);
         else memcpy(slotMemory(dev, slotA), src + off, nA);
         failed = send(slotA, off, nA);
