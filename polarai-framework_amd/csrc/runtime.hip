@@ -327,14 +327,14 @@ __attribute__((target("avx2"))) void streamCopyAvx2(char* dst, const char* src, 
 
 void copyOutOfSlot(void* dst, const void* src, size_t n);
 
-// Upload of one staging slot by the compute units instead of the DMA engine:
-// the slot is pinned host memory that the GPU can address, so a kernel on the
-// device's own queue reads it across the link and writes HBM.  Work that
+// Copy between a staging slot and device memory by the compute units instead of
+// the DMA engine: the slot is pinned host memory that the GPU can address, so a
+// kernel on the device's own queue moves the bytes across the link.  Work that
 // follows on the stream then starts as soon as the kernel retires; behind a
 // DMA-engine copy it waits for a signal from another engine, which costs
-// 10-15 us per upload in a graph whose kernels run for 2-10 us.
+// 10-15 us per transfer in a graph whose kernels run for 2-10 us.
 typedef float upload_v4 __attribute__((ext_vector_type(4)));
-__global__ __launch_bounds__(256) void uploadKernel(const upload_v4* src, upload_v4* dst, uint32_t vectors,
+__global__ __launch_bounds__(256) void slotCopyKernel(const upload_v4* src, upload_v4* dst, uint32_t vectors,
                                                     uint32_t tailBytes) {
   const uint32_t i = blockIdx.x * 256 + threadIdx.x;
   if (i < vectors) __builtin_nontemporal_store(__builtin_nontemporal_load(&src[i]), &dst[i]);
@@ -417,7 +417,7 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
         hipError_t e;
         if (!twoThreads && (reinterpret_cast<uintptr_t>(dst + off) & 15u) == 0) {
           const uint32_t vectors = static_cast<uint32_t>(n / 16), tail = static_cast<uint32_t>(n % 16);
-          hipLaunchKernelGGL(uploadKernel, dim3(vectors / 256 + 1), dim3(256), 0, dev->stream,
+          hipLaunchKernelGGL(slotCopyKernel, dim3(vectors / 256 + 1), dim3(256), 0, dev->stream,
                              reinterpret_cast<const upload_v4*>(slotMemory(dev, slot)),
                              reinterpret_cast<upload_v4*>(dst + off), vectors, tail);
           e = hipGetLastError();
@@ -517,8 +517,16 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
         failed = acquireSlot(dev, &slot);
         if (failed != hipSuccess) break;
         slots[c % kSlots] = slot;
-        failed = hipMemcpyAsync(slotMemory(dev, slot), static_cast<const char*>(src_device) + off, n,
-                                hipMemcpyDeviceToHost, dev->stream);
+        const char* from = static_cast<const char*>(src_device) + off;
+        if (!twoThreads && (reinterpret_cast<uintptr_t>(from) & 15u) == 0) {
+          const uint32_t vectors = static_cast<uint32_t>(n / 16), tail = static_cast<uint32_t>(n % 16);
+          hipLaunchKernelGGL(slotCopyKernel, dim3(vectors / 256 + 1), dim3(256), 0, dev->stream,
+                             reinterpret_cast<const upload_v4*>(from),
+                             reinterpret_cast<upload_v4*>(slotMemory(dev, slot)), vectors, tail);
+          failed = hipGetLastError();
+        } else {
+          failed = hipMemcpyAsync(slotMemory(dev, slot), from, n, hipMemcpyDeviceToHost, dev->stream);
+        }
         if (failed != hipSuccess) break;
         failed = hipEventRecord(dev->slotEvent[slot], dev->stream);
         if (failed != hipSuccess) break;
