@@ -94,9 +94,11 @@ int polar_hip_pool_get_stats(polar_hip_device* dev, polar_hip_pool_stats* out);
  *  src/backend/generic/runtime/sycl/SYCLDevice.h:81-112): ordered after all
  * work already enqueued on the device.  copy_to_host is complete when the call
  * returns.  copy_to_device has consumed src_host when it returns (the caller
- * may reuse it at once); for transfers of up to 4 MiB the DMA into dst_device
- * may still be in flight on the device's stream, where every later kernel,
- * copy and event of this library is ordered behind it. */
+ * may reuse it at once: the bytes were copied into pinned staging memory); the
+ * transfer into dst_device may still be in flight on the device's stream,
+ * where every later kernel, copy and event of this library is ordered behind
+ * it.  Transfers of 8 MiB and more use a second host thread of the library
+ * for half of the host-side copying. */
 int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
                              const void* src_host, uint64_t bytes);
 int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
@@ -216,7 +218,8 @@ int polar_hip_fsoftmax(polar_hip_device* dev, const float* in, float* out,
  * capture, tight serving loops, harnesses that forbid hipMalloc).  Same kernels
  * and same result, bit for bit, as polar_hip_fsoftmax; the partial sums go to
  * an array in the library's device data segment (256 KiB + 256 B per GPU, held
- * until the process ends) instead of a pool block.  n is limited to 2^31
+ * until the process ends) instead of the workspace block that the device
+ * allocates when it is opened.  n is limited to 2^31
  * elements; more returns POLAR_HIP_ERR_INVALID.  All calls on one GPU share
  * that array: calls that overlap on one GPU (two host threads, or two devices
  * handles opened on the same ordinal) race on it. */
