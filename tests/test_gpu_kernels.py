@@ -249,6 +249,43 @@ def test_matmul_short_contraction_tall_and_wide(dev, ta, tb, mnk):
         o.set_threads(1)
 
 
+NARROW_SHAPES = [(256, 10, 784), (784, 10, 256), (10, 256, 784), (16, 1000, 333), (1000, 16, 16), (64, 1, 5000),
+                 (65, 3, 4096), (70, 9, 4097), (5000, 7, 129), (8, 70000, 40), (70000, 5, 200), (300, 16, 17)]
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("mnk", NARROW_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_narrow_result(dev, ta, tb, mnk):
+    """One output dimension of at most 16 (a classifier's logits), either
+    operand in the narrow role, contractions from 16 to 5000: the planner's
+    small tiles and split-K plans.  Integer data (exact in any summation order)
+    with misaligned bases and a guard region, then random data against the
+    oracle."""
+    m, n, k = mnk
+    _say("narrow matmul", ta, tb, mnk)
+    rng = np.random.default_rng(m * 11 + n * 1013 + k + 2 * ta + tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    o.set_threads(o.hw_threads())
+    try:
+        a = rng.integers(-4, 5, sa).astype(np.float32)
+        b = rng.integers(-4, 5, sb).astype(np.float32)
+        da, db, dc = dev.array(a, 1), dev.array(b, 3), dev.empty(m * n + 64, 2)
+        dev.ffill(-7.0, dc, m * n + 64)
+        dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+        got = dc.download()
+        assert np.array_equal(got[:m * n].reshape(m, n), o.fmatmul(ta, tb, a, b))
+        assert np.all(got[m * n:] == -7.0)                 # nothing written past the end
+        for t in (da, db, dc):
+            t.free()
+        a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+        got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+        assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+        assert np.array_equal(got, _matmul_device(dev, ta, tb, a, b, m, n, k))   # repeatable
+    finally:
+        o.set_threads(1)
+
+
 SPLIT_K_SHAPES = [(33, 127, 4099), (33, 127, 65536), (256, 10, 784), (10, 256, 2051), (64, 64, 8192),
                   (130, 70, 3000), (1024, 1024, 4096)]
 
@@ -554,7 +591,7 @@ def test_pool_bit_exact(dev, shape, window, stride):
 # ---- extended (fused) builtins ----------------------------------------------------
 
 FUSED_SHAPES = [(256, 10, 784), (64, 64, 64), (33, 127, 4096), (300, 257, 129), (1024, 1024, 512), (5, 3, 0),
-                (2050, 33, 127), (40, 1500, 30)]
+                (2050, 33, 127), (40, 1500, 30), (784, 10, 256), (12, 300, 100)]
 
 
 @pytest.mark.parametrize("mnk", FUSED_SHAPES)
