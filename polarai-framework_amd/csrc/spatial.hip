@@ -26,8 +26,11 @@
 //    that the reads stay conflict-free, 16-byte staging loads), no LDS at all
 //    (a lane fetching its own KW+3 inputs per tap row: 98-110 us), a resident
 //    grid of groups that prefetch their next band into registers while they
-//    compute (116 us in row-major band order, 152 us walking down strips),
-//    16 or more rows per band (96-115 us); 8 to 12 rows measure the same.
+//    compute (116 us in row-major band order, 152 us walking down strips), a
+//    window per wave instead of per group, without any group barrier and with
+//    the first output rows computed while the later window rows are still in
+//    flight (105-142 us for 2-8 rows per wave), 16 or more rows per band
+//    (96-115 us); 8 to 12 rows measure the same.
 //  * fpool reads its windows straight from memory: with stride >= window each
 //    input element is used once, and the lanes of a wave walk consecutive
 //    windows, so the lines they touch are consumed completely by that wave.
