@@ -445,7 +445,8 @@ def bench_ceilings(args, n):
     best = max(out["read_only"].values(), key=lambda v: v["GB/s"])
     out["read_only"]["best_GB/s"] = best["GB/s"]
     names = {0: "32x256 tile, 1024 lanes", 1: "32x128 tile, 512 lanes", 2: "32x128 tile, 256 lanes",
-             3: "64x256 tile, 1024 lanes", 4: "32x64 tile, 256 lanes"}
+             3: "64x256 tile, 1024 lanes", 4: "32x64 tile, 256 lanes",
+             5: "128x64 tile, 512 lanes (512-byte chunks per output row)"}
     orders = {0: "row tiles fastest", 1: "column tiles fastest", 2: "column-tile range per XCD"}
     nbytes = 8 * T_ROWS * T_COLS
     for variant in names:

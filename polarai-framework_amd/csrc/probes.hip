@@ -264,12 +264,13 @@ int polar_probe_read(uint64_t n, int unroll, int sets, int warm, int reps, float
 
 // The memory pattern of a tiled rows x cols fp32 transpose.  variant selects
 // the tile: 0 = 32 x 256 (1024 lanes), 1 = 32 x 128 (512 lanes), 2 = 32 x 128
-// (256 lanes), 3 = 64 x 256 (1024 lanes), 4 = 32 x 64 (256 lanes); order: 0 =
+// (256 lanes), 3 = 64 x 256 (1024 lanes), 4 = 32 x 64 (256 lanes), 5 = 128 x 64
+// (512 lanes: 512-byte chunks per output row); order: 0 =
 // row tiles fastest, 1 = column tiles fastest, 2 = a contiguous range of column
 // tiles per XCD.  Bytes per launch: 8 rows cols.
 int polar_probe_transpose_pattern(uint32_t rows, uint32_t cols, int variant, int order, int sets,
                                   int warm, int reps, float* us) {
-  if (rows == 0 || cols == 0 || variant < 0 || variant > 4 || order < 0 || order > 2 || sets < 1 ||
+  if (rows == 0 || cols == 0 || variant < 0 || variant > 5 || order < 0 || order > 2 || sets < 1 ||
       reps < 1 || uint64_t(rows) * cols >= (1ull << 31))
     return hipErrorInvalidValue;
   Buffers mem;
@@ -290,7 +291,8 @@ int polar_probe_transpose_pattern(uint32_t rows, uint32_t cols, int variant, int
     case 1: launchPattern<32, 128, 512>(st.s, e0, e1, in, out, rows, cols, order); break;
     case 2: launchPattern<32, 128, 256>(st.s, e0, e1, in, out, rows, cols, order); break;
     case 3: launchPattern<64, 256, 1024>(st.s, e0, e1, in, out, rows, cols, order); break;
-    default: launchPattern<32, 64, 256>(st.s, e0, e1, in, out, rows, cols, order); break;
+    case 4: launchPattern<32, 64, 256>(st.s, e0, e1, in, out, rows, cols, order); break;
+    default: launchPattern<128, 64, 512>(st.s, e0, e1, in, out, rows, cols, order); break;
     }
   });
 }
