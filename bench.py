@@ -419,7 +419,8 @@ def bench_ceilings(args, n):
             raise RuntimeError(f"{fn.__name__} failed with hipError {status}")
         return float(np.mean(list(us)))
 
-    lib.polar_probe_streams.argtypes = [C.c_int, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
+    lib.polar_probe_streams.argtypes = [C.c_int, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                        C.POINTER(C.c_float)]
     lib.polar_probe_read.argtypes = [C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
     lib.polar_probe_transpose_pattern.argtypes = [C.c_uint32, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int,
                                                   C.c_int, C.POINTER(C.c_float)]
@@ -428,7 +429,7 @@ def bench_ceilings(args, n):
     for reads, like in ((0, "ffill"), (1, "fcopy frelu fsigmoid fconv2d"), (2, "fadd fmul fdivide flogloss"),
                         (4, "fpool 2x2 (4 reads per write)")):
         for ranges in (0, 1):
-            t = run(lib.polar_probe_streams, reads, n, ranges)
+            t = run(lib.polar_probe_streams, reads, n, ranges, 0, 0)
             gbs = 4 * n * (reads + 1) / (t * 1e-6) / 1e9
             order = "a contiguous eighth per XCD" if ranges else "pieces dealt round-robin to the XCDs"
             out["streams"][f"{reads}R+1W, {order}"] = {"us": round(t, 2), "GB/s": round(gbs, 1),
@@ -436,6 +437,15 @@ def bench_ceilings(args, n):
                                                        "pattern_of": like}
             log(f"probe {reads}R+1W streams, {order}: {t:7.1f} us  {gbs:7.1f} GB/s  "
                 f"{100 * gbs / HBM_PEAK_GBS:5.1f}%   ({like})")
+    # a copy whose output is off the line / 16-byte grid: what stores that straddle lines cost
+    out["misaligned_copy"] = {}
+    for shift, plain in ((0, 1), (4, 0), (4, 1), (2, 0), (2, 1)):
+        t = run(lib.polar_probe_streams, 1, n, 0, shift, plain)
+        gbs = 8 * n / (t * 1e-6) / 1e9
+        label = f"output {4 * shift} B behind a line boundary, {'plain' if plain else 'write-through streaming'} stores"
+        out["misaligned_copy"][label] = {"us": round(t, 2), "GB/s": round(gbs, 1),
+                                         "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+        log(f"probe copy, {label}: {t:7.1f} us  {gbs:7.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}%")
     for unroll in (2, 4, 8, 16):
         t = run(lib.polar_probe_read, n, unroll)
         gbs = 4 * n / (t * 1e-6) / 1e9
@@ -461,7 +471,7 @@ def bench_ceilings(args, n):
     out["transpose_pattern"]["best_GB/s"] = best["GB/s"]
     # the plain copy of the transpose's byte count
     nt = (T_ROWS * T_COLS) // 4 * 4
-    t = run(lib.polar_probe_streams, 1, nt, 0)
+    t = run(lib.polar_probe_streams, 1, nt, 0, 0, 0)
     out["copy_of_transpose_bytes"] = {"us": round(t, 2), "GB/s": round(8 * nt / (t * 1e-6) / 1e9, 1)}
     log(f"probe copy of {8 * nt} bytes: {t:7.1f} us  {8 * nt / (t * 1e-6) / 1e9:7.1f} GB/s")
     return out

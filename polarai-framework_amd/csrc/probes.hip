@@ -95,7 +95,8 @@ struct StreamPointers {
   v4f* out;
 };
 template <int READS, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void streamsKernel(StreamPointers p, uint64_t n4, int xcdRanges) {
+__global__ __launch_bounds__(BLOCK) void streamsKernel(StreamPointers p, uint64_t n4, int xcdRanges,
+                                                       int plainStores) {
   // xcdRanges: the groups of one XCD (ids equal modulo 8) take a contiguous
   // eighth of the streams instead of every eighth piece
   uint32_t group = blockIdx.x;
@@ -113,16 +114,21 @@ __global__ __launch_bounds__(BLOCK) void streamsKernel(StreamPointers p, uint64_
   for (int s = 0; s < READS; ++s)
 #pragma unroll
     for (int c = 0; c < 4; ++c) acc[c] = v[s][c] > acc[c] ? v[s][c] : acc[c];
-  asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(&p.out[i]), "v"(acc) : "memory");
+  // the output may start off a 16-byte boundary (see polar_probe_streams)
+  typedef float v4fu __attribute__((ext_vector_type(4), aligned(4)));
+  if (plainStores)
+    *reinterpret_cast<v4fu*>(&p.out[i]) = acc;
+  else
+    asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" : : "v"(&p.out[i]), "v"(acc) : "memory");
 }
 
 template <int READS, int BLOCK>
 void launchStreams(hipStream_t s, hipEvent_t e0, hipEvent_t e1, const StreamPointers& p, uint64_t n4,
-                   int xcdRanges) {
+                   int xcdRanges, int plainStores) {
   unsigned grid = static_cast<unsigned>((n4 + BLOCK - 1) / BLOCK);
   if (xcdRanges) grid = (grid + 7) / 8 * 8;
   hipExtLaunchKernelGGL((streamsKernel<READS, BLOCK>), dim3(grid), dim3(BLOCK), 0, s, e0, e1, 0, p, n4,
-                        xcdRanges);
+                        xcdRanges, plainStores);
 }
 
 // ---- read only: every lane sums UNROLL 16-byte loads, one float per group ---
@@ -206,9 +212,15 @@ extern "C" {
 // floats (reads in 0..4; n a multiple of 4), every stream an allocation of its
 // own; groups of 128 lanes, 256 for reads == 0 (the builtins' shapes).  Bytes
 // per launch: 4n(reads + 1).  xcdRanges != 0: each XCD works through a
-// contiguous eighth of every stream.
-int polar_probe_streams(int reads, uint64_t n, int xcdRanges, int sets, int warm, int reps, float* us) {
-  if (reads < 0 || reads > 4 || n % 4 != 0 || n == 0 || sets < 1 || reps < 1) return hipErrorInvalidValue;
+// contiguous eighth of every stream.  outShiftFloats: the output starts that
+// many floats behind a 128-byte boundary, so that a wave's 16-byte stores
+// straddle lines (and 16-byte boundaries, if not a multiple of 4).  plainStores:
+// ordinary cacheable stores instead of the write-through streaming ones.
+int polar_probe_streams(int reads, uint64_t n, int xcdRanges, int outShiftFloats, int plainStores, int sets,
+                        int warm, int reps, float* us) {
+  if (reads < 0 || reads > 4 || n % 4 != 0 || n == 0 || sets < 1 || reps < 1 || outShiftFloats < 0 ||
+      outShiftFloats > 31)
+    return hipErrorInvalidValue;
   Buffers mem;
   Stream st;
   PROBE_TRY(hipSetDevice(0));
@@ -221,17 +233,19 @@ int polar_probe_streams(int reads, uint64_t n, int xcdRanges, int sets, int warm
       PROBE_TRY(mem.add(n * 4, &b));
       ptrs[k].in[s] = static_cast<const v4f*>(b);
     }
-    PROBE_TRY(mem.add(n * 4, reinterpret_cast<void**>(&ptrs[k].out)));
+    void* o = nullptr;
+    PROBE_TRY(mem.add(n * 4 + 128, &o));
+    ptrs[k].out = reinterpret_cast<v4f*>(static_cast<float*>(o) + outShiftFloats);
   }
   const uint64_t n4 = n / 4;
   return timeLaunches(st.s, warm, reps, us, [&](int i, hipEvent_t e0, hipEvent_t e1) {
     const StreamPointers& p = ptrs[i % sets];
     switch (reads) {
-    case 0: launchStreams<0, 256>(st.s, e0, e1, p, n4, xcdRanges); break;
-    case 1: launchStreams<1, 128>(st.s, e0, e1, p, n4, xcdRanges); break;
-    case 2: launchStreams<2, 128>(st.s, e0, e1, p, n4, xcdRanges); break;
-    case 3: launchStreams<3, 128>(st.s, e0, e1, p, n4, xcdRanges); break;
-    default: launchStreams<4, 128>(st.s, e0, e1, p, n4, xcdRanges); break;
+    case 0: launchStreams<0, 256>(st.s, e0, e1, p, n4, xcdRanges, plainStores); break;
+    case 1: launchStreams<1, 128>(st.s, e0, e1, p, n4, xcdRanges, plainStores); break;
+    case 2: launchStreams<2, 128>(st.s, e0, e1, p, n4, xcdRanges, plainStores); break;
+    case 3: launchStreams<3, 128>(st.s, e0, e1, p, n4, xcdRanges, plainStores); break;
+    default: launchStreams<4, 128>(st.s, e0, e1, p, n4, xcdRanges, plainStores); break;
     }
   });
 }
