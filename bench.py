@@ -395,6 +395,13 @@ def bench_next_builtins(dev, dx, n, args):
     dpools = [dev.empty((h // 2) * (w // 2)) for _ in range(R)]
     ms = time_kernel(dev, lambda i: dev.fpool(dimgs[i % R], dpools[i % R], h, w, (2, 2), (2, 2)), args.warmup, args.steps)
     report("fpool", f"{h}x{w} image, max, window 2x2, stride 2x2", ms, 4 * (h * w + (h // 2) * (w // 2)))
+    # an overlapping window (the common CNN pooling): the staged kernel
+    oh3, ow3 = (h - 3) // 2 + 1, (w - 3) // 2 + 1
+    dpool3 = [dev.empty(oh3 * ow3) for _ in range(R)]
+    ms = time_kernel(dev, lambda i: dev.fpool(dimgs[i % R], dpool3[i % R], h, w, (3, 3), (2, 2)), args.warmup, args.steps)
+    report("fpool_3x3_stride2", f"{h}x{w} image, max, window 3x3, stride 2x2", ms, 4 * (h * w + oh3 * ow3))
+    for t in dpool3:
+        t.free()
     got = dpools[0].download((h // 2, w // 2))[:8]
     assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
     for t in dimgs + dpools + [dk]:

@@ -40,7 +40,11 @@
 //    Short bands are better (8192^2, 2x2, buffers rotated: 61.7 / 55.7 / 57.1 /
 //    58.7 / 60.3 us for 1 / 2 / 4 / 8 / 16 rows per group; four input streams
 //    merged into one output stream at full vector width take 54 us for the
-//    same bytes).
+//    same bytes).  Every other window and stride whose band fits 24 KB of LDS
+//    is staged like the convolution (poolStagedKernel; 8192^2, rotated: 3x3
+//    stride 2 148 -> 78-83 us, 3x3 stride 1 430 -> 119 us, 2x2 stride 1 281 ->
+//    91 us against one vector-memory instruction per tap before); larger windows
+//    fall back to taps from memory.
 #include "internal.h"
 
 using namespace polar_hip_detail;
@@ -54,6 +58,8 @@ constexpr int kLine = 32;     // floats per 128-byte line
 constexpr int kConvRows = 12; // output rows per fconv2d work-group
 constexpr int kPoolRows = 2;  // output rows per fpool work-group
 constexpr uint32_t kMaxConvLds = 64 * 1024;
+constexpr uint32_t kMaxPoolLds = 24 * 1024; // window of the staged fpool kernel: six groups per CU
+constexpr uint32_t kPoolStagedRows = 12;    // output rows per group of that kernel, at most
 
 // Work-group id -> tile index such that each XCD (ids equal modulo 8 share
 // one) works through a contiguous range of tiles: neighbouring tiles, which
@@ -292,6 +298,109 @@ __global__ __launch_bounds__(kSegment) void poolSquareKernel(PoolArgs p) {
   }
 }
 
+// Any window and stride, staged: the input window of a band of output rows goes
+// through LDS once (as in fconv2d), and the taps are read from there.  Reading
+// every tap from memory, as poolKernel does, costs a vector-memory instruction
+// per tap and output: 3x3 windows at stride 1 or 2 ran at 16-28 % of the HBM
+// rate that way, bound by the address unit, not by memory.
+// Window geometry for stride (s0, s1) and bandRows output rows: input rows
+// y0*s0 .. y0*s0 + (bandRows-1)*s0 + win0 - 1; input columns from
+// (ct*256 - 31)*s1 (the segment's leftmost possible output column) over
+// (256 + 31 - 1)*s1 + win1 columns.
+struct PoolStagedArgs {
+  PoolArgs pool;
+  uint32_t bandRows; // output rows per work-group
+  uint32_t pitch;    // window columns
+};
+
+// W0_/W1_ == 0: the window size comes from the arguments.
+template <int W0_, int W1_>
+__global__ __launch_bounds__(kSegment) void poolStagedKernel(PoolStagedArgs q) {
+  extern __shared__ float tile[];
+  const PoolArgs& p = q.pool;
+  const uint32_t win0 = W0_ ? W0_ : p.win0, win1 = W1_ ? W1_ : p.win1;
+  uint32_t tileIdx;
+  if (!tileOfGroup(p.tiles, &tileIdx)) return; // before any barrier
+  const uint32_t ct = tileIdx % p.colTiles, rt = tileIdx / p.colTiles;
+  const uint32_t y0 = rt * q.bandRows;
+  const uint32_t rowsOut = p.OH - y0 < q.bandRows ? p.OH - y0 : q.bandRows;
+  const uint32_t rowsIn = (rowsOut - 1) * p.stride0 + win0; // all inside the input
+  const uint32_t pitch = q.pitch;
+  const int64_t x0 = (int64_t(ct) * kSegment - (kLine - 1)) * int64_t(p.stride1); // may be negative
+  const uint32_t t = threadIdx.x;
+
+  // Stage: lane t takes window elements t, t+256, ... in row-major order
+  // (pitch > 256, so a step of 256 wraps to the next row at most once).
+  // Stage: lane t takes window elements t, t+256, ... in row-major order
+  // (pitch > 256, so a step of 256 wraps to the next row at most once), eight
+  // loads at a time (the whole window's loads at once, up to 24: 10-25 %
+  // slower; 4 or 12 at a time: within a few per cent either way).
+  const uint32_t total = rowsIn * pitch;
+  constexpr int kBatch = 8;
+  const bool inside = x0 >= 0 && x0 + pitch <= int64_t(p.W);
+  uint32_t col = t;
+  const float* src = p.in + uint64_t(y0) * p.stride0 * p.W + x0 + t; // never dereferenced outside the image
+  for (uint32_t idx = t; idx < total; idx += kSegment * kBatch) {
+    float v[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int64_t xi = x0 + col;
+      const bool ok = idx + u * kSegment < total && (inside || (xi >= 0 && xi < int64_t(p.W)));
+      v[u] = ok ? *src : 0.0f;
+      col += kSegment;
+      src += kSegment;
+      if (col >= pitch) {
+        col -= pitch;
+        src += int64_t(p.W) - pitch;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+      if (idx + u * kSegment < total) tile[idx + u * kSegment] = v[u];
+  }
+  __syncthreads();
+
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(t / 64), lane = t % 64;
+  const int32_t ow = int32_t(p.OW);
+  for (uint32_t r = wave; r < rowsOut; r += kSegment / 64) {
+    const uint32_t y = y0 + r;
+    const uint32_t shift = rowShift(y, p.OW, p.outPhase);
+    float* const rowOut = p.out + uint64_t(y) * p.OW;
+    // the lane's first output of the row; its others are 64 outputs further on each
+    const float* corner = tile + r * p.stride0 * pitch + (uint32_t(kLine - 1) - shift + lane) * p.stride1;
+    const int32_t x = int32_t(ct * kSegment + lane) - int32_t(shift);
+    const uint32_t step = 64 * p.stride1;
+    // utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:50-52,74-76: starts
+    // at -10e5, strict ordered greater-than, rows outer / columns inner
+    float best[4] = {-10e5f, -10e5f, -10e5f, -10e5f};
+    if constexpr (W0_ != 0) {
+#pragma unroll
+      for (int a = 0; a < W0_; ++a)
+#pragma unroll
+        for (int b = 0; b < W1_; ++b)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float v = corner[a * pitch + b + j * step];
+            best[j] = v > best[j] ? v : best[j];
+          }
+    } else {
+      for (uint32_t a = 0; a < win0; ++a)
+        for (uint32_t b = 0; b < win1; ++b) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float v = corner[a * pitch + b + j * step];
+            best[j] = v > best[j] ? v : best[j];
+          }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int32_t xj = x + 64 * j;
+      if (xj >= 0 && xj < ow) streamStore(best[j], rowOut + xj);
+    }
+  }
+}
+
 uint32_t phaseOf(const float* out) {
   return static_cast<uint32_t>((reinterpret_cast<uintptr_t>(out) / sizeof(float)) % kLine);
 }
@@ -385,6 +494,31 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
     return p.win0 == w && p.win1 == w && p.stride0 == w && p.stride1 == w && p.W % w == 0 &&
            reinterpret_cast<uintptr_t>(in) % (sizeof(float) * w) == 0;
   };
+  if (!square(2) && !square(4)) {
+    // staged kernel if a band of at least one output row fits the LDS budget
+    PoolStagedArgs q;
+    q.pool = p;
+    q.pitch = (kSegment + kLine - 2) * p.stride1 + p.win1;
+    const uint64_t floats = kMaxPoolLds / sizeof(float);
+    const uint64_t rowsFit = floats / q.pitch; // input rows
+    if (rowsFit >= p.win0 && uint64_t(p.H) * p.W < (1ull << 40)) {
+      uint64_t band = (rowsFit - p.win0) / p.stride0 + 1;
+      if (band > kPoolStagedRows) band = kPoolStagedRows;
+      q.bandRows = static_cast<uint32_t>(band);
+      const uint64_t stagedTiles = uint64_t(p.colTiles) * ((p.OH + q.bandRows - 1) / q.bandRows);
+      POLAR_HIP_REQUIRE(stagedTiles < (1ull << 31) - kXcds, "tensor too large for one launch");
+      q.pool.tiles = static_cast<uint32_t>(stagedTiles);
+      const uint32_t ldsBytes = static_cast<uint32_t>(
+          (uint64_t(q.bandRows - 1) * p.stride0 + p.win0) * q.pitch * sizeof(float));
+      auto staged = p.win0 == 2 && p.win1 == 2   ? poolStagedKernel<2, 2>
+                    : p.win0 == 3 && p.win1 == 3 ? poolStagedKernel<3, 3>
+                    : p.win0 == 5 && p.win1 == 5 ? poolStagedKernel<5, 5>
+                                                 : poolStagedKernel<0, 0>;
+      POLAR_HIP_TRY(launchKernelLds(dev, staged, dim3(static_cast<unsigned>(paddedGrid(stagedTiles))),
+                                    dim3(kSegment), ldsBytes, q));
+      return POLAR_HIP_OK;
+    }
+  }
   auto fn = square(2) ? poolSquareKernel<2> : square(4) ? poolSquareKernel<4> : poolKernel;
   POLAR_HIP_TRY(launchKernel(dev, fn, dim3(static_cast<unsigned>(grid)), dim3(kSegment), p));
   return POLAR_HIP_OK;
