@@ -568,7 +568,13 @@ POOL_CASES = [((4, 4), (2, 2), (2, 2)), ((100, 257), (2, 2), (2, 2)), ((101, 333
               ((257, 1031), (2, 2), (2, 2)), ((16, 4100), (4, 4), (4, 4)), ((30, 30), (5, 5), (7, 7)),
               # even widths: the vector-load kernel for non-overlapping 2x2 / 4x4 windows, ragged edges
               ((101, 334), (2, 2), (2, 2)), ((37, 1030), (2, 2), (2, 2)), ((2, 2), (2, 2), (2, 2)),
-              ((19, 6), (2, 2), (2, 2)), ((9, 516), (4, 4), (4, 4)), ((67, 2052), (4, 4), (4, 4))]
+              ((19, 6), (2, 2), (2, 2)), ((9, 516), (4, 4), (4, 4)), ((67, 2052), (4, 4), (4, 4)),
+              # the staged kernel: overlapping windows, strides beyond the window, several column tiles and
+              # bands, a ragged last band, widths around one segment; then windows too large for its LDS budget
+              ((300, 1200), (3, 3), (1, 1)), ((133, 777), (2, 2), (1, 1)), ((200, 2100), (3, 3), (2, 2)),
+              ((97, 1500), (5, 5), (2, 2)), ((64, 900), (2, 3), (4, 5)), ((41, 290), (3, 3), (3, 3)),
+              ((40, 258), (7, 2), (1, 1)), ((300, 40), (3, 5), (2, 1)), ((13, 4000), (13, 1), (1, 2)),
+              ((120, 600), (30, 30), (5, 5)), ((60, 700), (3, 200), (2, 100))]
 
 
 @pytest.mark.parametrize("shape,window,stride", POOL_CASES)
