@@ -51,7 +51,8 @@ TRAFFIC_KERNELS = {  # operation -> name fragments of the kernels one call launc
     "fadd": ["<AddOp,"], "fmul": ["<MulOp,"], "fdivide": ["<DivOp,"], "fsigmoid": ["<SigmoidOp,"],
     "fcopy": ["<CopyOp,"], "ffill": ["<FillOp,"], "flogloss": ["<LogLossOp,"], "fmulconcat": ["<ScaleOp,"],
     "frelu": ["<ReluOp,"], "fsoftmax": ["expSumKernel", "finishSumKernel", "<SoftmaxScaleOp,"],
-    "ftranspose": ["transpose"], "fmatmul": ["matmulKernel<"], "fconv2d": ["conv2d"], "fpool": ["pool"],
+    "ftranspose": ["transpose"], "fmatmul": ["matmulKernel<"], "fconv2d": ["conv2d"], "fpool": ["poolSquareKernel"],
+    "fpool_3x3_stride2": ["poolStagedKernel"],
 }
 
 
