@@ -104,6 +104,26 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
 int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
                            const void* src_device, uint64_t bytes);
 
+/* ---- host memory the GPU can address ----------------------------------------
+ * No counterpart in the reference, whose host-side tensor storage is new[]
+ * (src/backend/generic/lib/allocators/TrivialAllocator.hpp:23-93).  A caller
+ * that keeps its host copies of tensors in blocks from polar_hip_host_alloc
+ * (pinned memory) saves the staging copy of every transfer: the two copy
+ * calls above recognise a host pointer inside such a block and move the bytes
+ * directly between it and device memory.
+ * Consequence for copy_to_device from such a block: the call returns with the
+ * transfer queued, not with the source consumed.  Before the host WRITES the
+ * block again it calls polar_hip_host_quiesce, which returns once every queued
+ * transfer out of the block has completed.  That costs nothing when the caller
+ * has meanwhile waited for an event recorded behind the transfer
+ * (polar_hip_event_synchronize / _query, polar_hip_device_synchronize): the
+ * library notes how far the stream has got.  Otherwise it waits for all work
+ * the stream holds.  polar_hip_host_free quiesces by itself.  The blocks are process-wide: they
+ * outlive the device handle they were allocated through. */
+int polar_hip_host_alloc(polar_hip_device* dev, uint64_t bytes, void** ptr);
+int polar_hip_host_free(void* ptr);
+int polar_hip_host_quiesce(void* ptr);
+
 /* ---- events -------------------------------------------------------------------
  * Stand in for the native event inside the reference's Event objects
  * (src/backend/generic/runtime/cuda/CudaEvent.cpp:18-31,

@@ -66,6 +66,9 @@ SIGNATURES = {
     "polar_hip_pool_get_stats": (_i, [_vp, C.POINTER(PoolStats)]),
     "polar_hip_copy_to_device": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_copy_to_host": (_i, [_vp, _vp, _vp, _u64]),
+    "polar_hip_host_alloc": (_i, [_vp, _u64, C.POINTER(_vp)]),
+    "polar_hip_host_free": (_i, [_vp]),
+    "polar_hip_host_quiesce": (_i, [_vp]),
     "polar_hip_event_record": (_i, [_vp, C.POINTER(_vp)]),
     "polar_hip_event_synchronize": (_i, [_vp]),
     "polar_hip_event_query": (_i, [_vp, C.POINTER(_i)]),
@@ -236,6 +239,18 @@ class Device:
 
     def copy_to_host(self, dst_host, src, nbytes):
         _check(self.lib, self.lib.polar_hip_copy_to_host(self.handle, dst_host, src, nbytes))
+
+    def host_alloc(self, nbytes):
+        """Pinned host memory that the copy calls move to and from directly."""
+        p = _vp()
+        _check(self.lib, self.lib.polar_hip_host_alloc(self.handle, nbytes, C.byref(p)))
+        return p.value
+
+    def host_free(self, ptr):
+        _check(self.lib, self.lib.polar_hip_host_free(ptr))
+
+    def host_quiesce(self, ptr):
+        _check(self.lib, self.lib.polar_hip_host_quiesce(ptr))
 
     def pool_stats(self):
         st = PoolStats()

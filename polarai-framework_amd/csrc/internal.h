@@ -9,6 +9,7 @@
 #include <cstdarg>
 #include <condition_variable>
 #include <cstdint>
+#include <atomic>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -22,6 +23,10 @@
 struct polar_hip_event {
   polar_hip_device* dev;
   hipEvent_t ev;
+  // number of the last direct host-block transfer queued on the stream before
+  // this event was recorded (see polar_hip_device::directQueued); 0 for events
+  // attached to a kernel
+  uint64_t directStamp = 0;
 };
 
 // Second host thread of large device-to-host copies: the staging slots are
@@ -59,6 +64,10 @@ struct polar_hip_device {
   void* staging = nullptr;
   hipEvent_t slotEvent[8] = {};
   bool slotBusy[8] = {};
+  // a busy slot either has slotEvent recorded behind its transfer, or (small
+  // uploads) only the transfer's number in the directQueued sequence
+  bool slotEvented[8] = {};
+  uint64_t slotNumber[8] = {};
   int nextSlot = 0;
   DrainThread drain; // used under stagingMu
 
@@ -78,6 +87,18 @@ struct polar_hip_device {
   // call enqueues the kernels that share it.
   std::mutex workspaceMu;
   void* workspace = nullptr;
+  // Transfers queued directly out of or into blocks of polar_hip_host_alloc are
+  // numbered per device handle; directDone is the highest number known to be
+  // complete, learnt from whatever the caller waits for anyway (an event
+  // recorded behind the transfer, the whole stream), so that the blocks need no
+  // events of their own.  `serial` names this handle in the blocks' bookkeeping.
+  uint64_t serial = 0;
+  std::atomic<uint64_t> directQueued{0}, directDone{0};
+  void noteDirectDone(uint64_t number) {
+    uint64_t seen = directDone.load(std::memory_order_relaxed);
+    while (seen < number && !directDone.compare_exchange_weak(seen, number)) {
+    }
+  }
 };
 
 struct polar_hip_module {

@@ -12,6 +12,12 @@ namespace {
 thread_local char g_lastError[512] = "";
 void drainStop(DrainThread& d); // with the copy code below
 
+// Host blocks the GPU can address (polar_hip_host_alloc) and the open device
+// handles their queued transfers refer to.
+std::mutex g_hostMu;
+std::map<uint64_t, polar_hip_device*> g_openDevices; // by serial
+uint64_t g_nextSerial = 1;
+
 uint64_t roundBlock(uint64_t bytes) {
   // Small blocks: powers of two from 256 B.  Large blocks: multiples of 2 MiB,
   // so that tensors of nearly equal size share cached blocks.
@@ -118,6 +124,11 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
     delete d;
     return st;
   }
+  {
+    std::lock_guard<std::mutex> g(g_hostMu);
+    d->serial = g_nextSerial++;
+    g_openDevices.emplace(d->serial, d);
+  }
   *out = d;
   return POLAR_HIP_OK;
 }
@@ -126,6 +137,12 @@ int polar_hip_device_close(polar_hip_device* dev) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  {
+    // every transfer this handle queued out of a host block is complete now;
+    // a block that still names the handle finds it gone and takes that as done
+    std::lock_guard<std::mutex> g(g_hostMu);
+    g_openDevices.erase(dev->serial);
+  }
   for (auto& kv : dev->cached)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : dev->live) (void)hipFree(kv.first);
@@ -153,7 +170,9 @@ int polar_hip_device_get_info(polar_hip_device* dev,
 
 int polar_hip_device_synchronize(polar_hip_device* dev) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
+  const uint64_t queued = dev->directQueued.load();
   POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+  dev->noteDirectDone(queued);
   return POLAR_HIP_OK;
 }
 
@@ -286,8 +305,18 @@ hipError_t acquireSlot(polar_hip_device* dev, int* slot) {
   const int s = dev->nextSlot;
   dev->nextSlot = (s + 1) % kSlots;
   if (dev->slotBusy[s]) {
-    hipError_t e = hipEventSynchronize(dev->slotEvent[s]);
-    if (e != hipSuccess) return e;
+    if (dev->slotEvented[s]) {
+      hipError_t e = hipEventSynchronize(dev->slotEvent[s]);
+      if (e != hipSuccess) return e;
+    } else if (dev->directDone.load() < dev->slotNumber[s]) {
+      // a small upload left no event, and nothing the caller has waited for
+      // since tells that it is over: wait for what the stream holds now
+      const uint64_t queued = dev->directQueued.load();
+      hipError_t e = hipEventRecord(dev->slotEvent[s], dev->stream);
+      if (e == hipSuccess) e = hipEventSynchronize(dev->slotEvent[s]);
+      if (e != hipSuccess) return e;
+      dev->noteDirectDone(queued);
+    }
     dev->slotBusy[s] = false;
   }
   *slot = s;
@@ -394,6 +423,109 @@ void copyOutOfSlot(void* dst, const void* src, size_t n) {
 }
 } // namespace
 
+// ---- host blocks the GPU can address -----------------------------------------
+namespace {
+struct HostBlock {
+  uint64_t bytes = 0;
+  // the latest transfer queued directly out of or into the block: its number on
+  // the device handle `serial` (0: none outstanding)
+  uint64_t serial = 0, number = 0;
+};
+std::map<uintptr_t, HostBlock> g_hostBlocks; // by base address; g_hostMu
+
+// the block that holds [p, p + bytes), or null; g_hostMu held
+HostBlock* hostBlockOf(const void* p, uint64_t bytes) {
+  const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+  auto it = g_hostBlocks.upper_bound(a);
+  if (it == g_hostBlocks.begin()) return nullptr;
+  --it;
+  return a + bytes <= it->first + it->second.bytes ? &it->second : nullptr;
+}
+
+// Returns once the latest transfer queued on the block is complete.  Usually
+// that is already known: the caller has waited for an event recorded behind the
+// transfer (every launch of a graph is followed by one), and the device handle
+// has noted how far its stream had got.  Otherwise the whole stream is waited
+// for.  No event per transfer: a recorded event puts a marker packet between
+// the kernels, and waiting for an idle stream costs tens of microseconds.
+// g_hostMu held.
+hipError_t waitForBlock(HostBlock& b) {
+  if (b.number == 0) return hipSuccess;
+  auto it = g_openDevices.find(b.serial);
+  if (it != g_openDevices.end() && it->second->directDone.load() < b.number) {
+    polar_hip_device* dev = it->second;
+    const uint64_t queued = dev->directQueued.load();
+    const hipError_t e = hipStreamSynchronize(dev->stream);
+    if (e != hipSuccess) return e;
+    dev->noteDirectDone(queued);
+  }
+  b.number = 0;
+  return hipSuccess;
+}
+
+// Queue a transfer between a host block and device memory on dev's stream and
+// note it on the block.  g_hostMu held.
+hipError_t queueDirect(polar_hip_device* dev, HostBlock& b, void* dst, const void* src, uint64_t bytes,
+                       hipMemcpyKind kind) {
+  // another handle's transfer on the block first: one note per block
+  if (b.number != 0 && b.serial != dev->serial) {
+    const hipError_t w = waitForBlock(b);
+    if (w != hipSuccess) return w;
+  }
+  hipError_t e;
+  if (bytes < kTwoThreadBytes && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0) {
+    const uint32_t vectors = static_cast<uint32_t>(bytes / 16), tail = static_cast<uint32_t>(bytes % 16);
+    hipLaunchKernelGGL(slotCopyKernel, dim3(vectors / 256 + 1), dim3(256), 0, dev->stream,
+                       static_cast<const upload_v4*>(src), static_cast<upload_v4*>(dst), vectors, tail);
+    e = hipGetLastError();
+  } else {
+    e = hipMemcpyAsync(dst, src, bytes, kind, dev->stream);
+  }
+  if (e != hipSuccess) return e;
+  b.serial = dev->serial;
+  b.number = dev->directQueued.fetch_add(1) + 1; // after the launch: an event stamped with it is behind the transfer
+  return hipSuccess;
+}
+} // namespace
+
+int polar_hip_host_alloc(polar_hip_device* dev, uint64_t bytes, void** ptr) {
+  POLAR_HIP_REQUIRE(dev != nullptr && ptr != nullptr, "null argument");
+  *ptr = nullptr;
+  POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  void* p = nullptr;
+  POLAR_HIP_TRY(hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocPortable | hipHostMallocMapped));
+  std::lock_guard<std::mutex> g(g_hostMu);
+  HostBlock b;
+  b.bytes = bytes ? bytes : 1;
+  g_hostBlocks.emplace(reinterpret_cast<uintptr_t>(p), b);
+  *ptr = p;
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_host_free(void* ptr) {
+  if (ptr == nullptr) return POLAR_HIP_OK;
+  {
+    std::lock_guard<std::mutex> g(g_hostMu);
+    auto it = g_hostBlocks.find(reinterpret_cast<uintptr_t>(ptr));
+    if (it == g_hostBlocks.end())
+      return fail(POLAR_HIP_ERR_INVALID, "polar_hip_host_free: %p is not a block of polar_hip_host_alloc", ptr);
+    POLAR_HIP_TRY(waitForBlock(it->second));
+    g_hostBlocks.erase(it);
+  }
+  POLAR_HIP_TRY(hipHostFree(ptr));
+  return POLAR_HIP_OK;
+}
+
+int polar_hip_host_quiesce(void* ptr) {
+  if (ptr == nullptr) return POLAR_HIP_OK;
+  std::lock_guard<std::mutex> g(g_hostMu);
+  HostBlock* b = hostBlockOf(ptr, 1);
+  if (b == nullptr)
+    return fail(POLAR_HIP_ERR_INVALID, "polar_hip_host_quiesce: %p is not inside a block of polar_hip_host_alloc", ptr);
+  POLAR_HIP_TRY(waitForBlock(*b));
+  return POLAR_HIP_OK;
+}
+
 int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
                              const void* src_host, uint64_t bytes) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
@@ -401,6 +533,14 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
   POLAR_HIP_REQUIRE(dst_device != nullptr && src_host != nullptr,
                     "null buffer");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
+  {
+    // source inside a block of polar_hip_host_alloc: no staging
+    std::lock_guard<std::mutex> g(g_hostMu);
+    if (HostBlock* b = hostBlockOf(src_host, bytes)) {
+      POLAR_HIP_TRY(queueDirect(dev, *b, dst_device, src_host, bytes, hipMemcpyHostToDevice));
+      return POLAR_HIP_OK;
+    }
+  }
   {
     // The data is copied into pinned slots and sent from there, so the call
     // returns once the last DMA is queued and the caller may reuse its memory.
@@ -411,6 +551,12 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
     if (stagingReady(dev)) {
       const bool twoThreads = bytes >= kTwoThreadBytes;
       const uint64_t chunkBytes = twoThreads ? kSlotCapacity : kSlotBytes;
+      // Uploads of one or two chunks (graph inputs) record no event behind
+      // their slots: a recorded event is a marker packet between the kernels
+      // and a few microseconds of host time, and the slot is normally known to
+      // be free again from an event the caller waited for in the meantime (see
+      // acquireSlot).  Longer uploads reuse slots while they run and need them.
+      const bool evented = bytes > 2 * kSlotBytes;
       const char* src = static_cast<const char*>(src_host);
       char* dst = static_cast<char*>(dst_device);
       auto send = [&](int slot, uint64_t off, uint64_t n) -> hipError_t {
@@ -425,8 +571,12 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
           e = hipMemcpyAsync(dst + off, slotMemory(dev, slot), n, hipMemcpyHostToDevice, dev->stream);
         }
         if (e != hipSuccess) return e;
-        e = hipEventRecord(dev->slotEvent[slot], dev->stream);
-        if (e == hipSuccess) dev->slotBusy[slot] = true;
+        if (evented) e = hipEventRecord(dev->slotEvent[slot], dev->stream);
+        else dev->slotNumber[slot] = dev->directQueued.fetch_add(1) + 1;
+        if (e == hipSuccess) {
+          dev->slotBusy[slot] = true;
+          dev->slotEvented[slot] = evented;
+        }
         return e;
       };
       hipError_t failed = hipSuccess;
@@ -476,6 +626,17 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
                     "null buffer");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   {
+    // destination inside a block of polar_hip_host_alloc: written directly, and
+    // complete when the call returns (this handle's own earlier transfers out
+    // of the block are ahead of the new one on its stream)
+    std::lock_guard<std::mutex> g(g_hostMu);
+    if (HostBlock* b = hostBlockOf(dst_host, bytes)) {
+      POLAR_HIP_TRY(queueDirect(dev, *b, dst_host, src_device, bytes, hipMemcpyDeviceToHost));
+      POLAR_HIP_TRY(waitForBlock(*b));
+      return POLAR_HIP_OK;
+    }
+  }
+  {
     // Any size: at most kSlots chunk DMAs are in flight; a chunk is copied out
     // as soon as its event completes and its slot goes to the chunk kSlots
     // further on.  In a large transfer every second chunk is copied out by the
@@ -488,6 +649,7 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
     std::lock_guard<std::mutex> g(dev->stagingMu);
     if (stagingReady(dev)) {
       int slots[kSlots];
+      const uint64_t queuedBefore = dev->directQueued.load();
       const bool twoThreads = bytes >= kTwoThreadBytes;
       // per chunk this thread pays about 10 us of driver calls; with 512 KiB
       // chunks that alone capped a 256 MiB read-back at 24 GB/s
@@ -500,6 +662,7 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
         hipError_t e = hipEventSynchronize(dev->slotEvent[slot]);
         if (e != hipSuccess) return e;
         dev->slotBusy[slot] = false;
+        dev->noteDirectDone(queuedBefore); // ahead of this chunk on the stream
         if (twoThreads && (c & 1))
           drainPost(dev->drain, static_cast<char*>(dst_host) + off, slotMemory(dev, slot), n);
         else
@@ -531,6 +694,7 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
         failed = hipEventRecord(dev->slotEvent[slot], dev->stream);
         if (failed != hipSuccess) break;
         dev->slotBusy[slot] = true;
+        dev->slotEvented[slot] = true;
       }
       for (uint64_t c = chunks > lag ? chunks - lag : 0; c < chunks && failed == hipSuccess; ++c)
         failed = consume(c);
@@ -566,6 +730,7 @@ int polar_hip_event_record(polar_hip_device* dev, polar_hip_event** out) {
     std::lock_guard<std::mutex> g(dev->mu);
     dev->allEvents.push_back(e);
   }
+  e->directStamp = dev->directQueued.load();
   hipError_t err = hipEventRecord(e->ev, dev->stream);
   if (err != hipSuccess) {
     std::lock_guard<std::mutex> g(dev->mu);
@@ -584,12 +749,16 @@ int polar_hip_event_synchronize(polar_hip_event* evt) {
   const auto t0 = std::chrono::steady_clock::now();
   for (;;) {
     hipError_t e = hipEventQuery(evt->ev);
-    if (e == hipSuccess) return POLAR_HIP_OK;
+    if (e == hipSuccess) {
+      evt->dev->noteDirectDone(evt->directStamp);
+      return POLAR_HIP_OK;
+    }
     if (e != hipErrorNotReady) return failHip(e, "hipEventQuery");
     (void)hipGetLastError();
     if (std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(200)) break;
   }
   POLAR_HIP_TRY(hipEventSynchronize(evt->ev));
+  evt->dev->noteDirectDone(evt->directStamp);
   return POLAR_HIP_OK;
 }
 
@@ -597,6 +766,7 @@ int polar_hip_event_query(polar_hip_event* evt, int* done) {
   POLAR_HIP_REQUIRE(evt != nullptr && done != nullptr, "null argument");
   hipError_t e = hipEventQuery(evt->ev);
   if (e == hipSuccess) {
+    evt->dev->noteDirectDone(evt->directStamp);
     *done = 1;
   } else if (e == hipErrorNotReady) {
     (void)hipGetLastError();
@@ -644,6 +814,7 @@ int polar_hip_time_next_kernel(polar_hip_device* dev, polar_hip_event** start,
       dev->allEvents.push_back(e);
     }
   }
+  pair[0]->directStamp = pair[1]->directStamp = 0; // attached to a kernel, not recorded behind the stream
   dev->timeStart = *start = pair[0];
   dev->timeStop = *stop = pair[1];
   return POLAR_HIP_OK;
