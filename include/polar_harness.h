@@ -64,6 +64,14 @@ const char* polar_harness_device_name(polar_harness* h);
 int polar_harness_device_provider(polar_harness* h);
 int polar_harness_device_kind(polar_harness* h);
 
+/* Take the RAM-side blocks of tensors from the plugin's pinned host memory
+ * (its optional polarHostMemoryAllocate / Release / Quiesce symbols) instead
+ * of the heap, so that uploads and read-backs need no staging copy.  Call
+ * before the first tensor is allocated.  Returns -1 if the plugin does not
+ * export the three symbols (or for the mock device); 0 otherwise.  Off by
+ * default: the framework's own RAM layer uses the heap. */
+int polar_harness_use_plugin_host_memory(polar_harness* h);
+
 /* Reserve a tensor: returns its virtual address in the context's flat space
  * (first tensor at 1, each next one after the previous one's bytes, as
  * src/core/context/internal/ContextInternal.cpp:43-48). */

@@ -116,6 +116,20 @@ polarai::backend::generic::BackendAllocator* polar_rt_support_allocator_create()
 void polar_rt_support_allocator_destroy(polarai::backend::generic::BackendAllocator*);
 void polar_rt_support_register_device(polarai::backend::generic::BackendAllocator*,
                                       polarai::backend::generic::Device*);
+// Optional: where the allocator's RAM-side blocks come from.  With blocks the
+// device can address (a runtime plugin's pinned memory), Device::copyToDevice
+// and copyToHost need no staging copy.  `quiesce` is called before host code is
+// given access to a block (every lock of a record on the host device), so that
+// an upload the device still has queued out of the block is complete before the
+// host overwrites it; it may be null.  Set before the first tensor is allocated.
+// Without this call the blocks come from the heap, as the framework's do.
+struct polar_rt_host_memory {
+  void* (*allocate)(size_t bytes); // may return null: the heap is used for that block
+  void (*release)(void* block);
+  void (*quiesce)(void* block);
+};
+void polar_rt_support_set_host_memory(polarai::backend::generic::BackendAllocator*,
+                                      const polar_rt_host_memory* hooks);
 // The "host" device input nodes are routed to
 // (src/backend/generic/runtime/host/HostDevice.hpp:17-52).
 polarai::backend::generic::Device* polar_rt_support_host_device_create();

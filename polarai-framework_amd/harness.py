@@ -32,6 +32,7 @@ _vp, _u64, _i = C.c_void_p, C.c_uint64, C.c_int
 SIGNATURES = {
     "polar_harness_open": (_i, [C.c_char_p, _i, C.POINTER(_vp)]),
     "polar_harness_close": (None, [_vp]),
+    "polar_harness_use_plugin_host_memory": (_i, [_vp]),
     "polar_harness_device_count": (_i, [_vp]),
     "polar_harness_device_name": (C.c_char_p, [_vp]),
     "polar_harness_device_provider": (_i, [_vp]),
@@ -83,7 +84,10 @@ class Tensor:
 
 
 class Harness:
-    def __init__(self, plugin=LIB_PLUGIN, device_index=0):
+    def __init__(self, plugin=LIB_PLUGIN, device_index=0, plugin_host_memory=False):
+        """plugin_host_memory: keep the RAM side of every tensor in the plugin's pinned host
+        memory (polar_harness_use_plugin_host_memory); the default is the heap, as in the
+        framework's own RAM layer."""
         self.lib = load_library()
         if plugin is not None and not os.path.exists(plugin):
             raise FileNotFoundError(f"{plugin} is not built; run __graft_entry__.build()")
@@ -94,6 +98,9 @@ class Harness:
             raise RuntimeError(f"cannot open runtime plugin {plugin} (device {device_index})")
         self.h = h
         self._keep = []
+        if plugin_host_memory and self.lib.polar_harness_use_plugin_host_memory(h) != 0:
+            self.close()
+            raise RuntimeError(f"{plugin} does not export polarHostMemoryAllocate/Release/Quiesce")
 
     def close(self):
         if self.h is not None:

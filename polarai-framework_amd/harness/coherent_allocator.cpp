@@ -21,14 +21,25 @@ void fatalError(int code, const char* fmt, ...) {
 
 // ---- RAM layer ----------------------------------------------------------------
 
+void RamLayer::freeBlock(Block& b) {
+  if (b.provided) mRelease(b.mem);
+  else std::free(b.mem);
+  b.mem = nullptr;
+}
+
 RamLayer::~RamLayer() {
-  for (auto& kv : mBlocks) std::free(kv.second.mem);
+  for (auto& kv : mBlocks) freeBlock(kv.second);
 }
 
 void RamLayer::allocate(MemoryRecord record) {
   if (mBlocks.count(record.virtualAddress)) return;
   Block b;
-  b.mem = std::aligned_alloc(64, (record.allocationSize + 63) / 64 * 64 + 64);
+  const size_t bytes = (record.allocationSize + 63) / 64 * 64 + 64;
+  if (mAllocate != nullptr && mRelease != nullptr) {
+    b.mem = mAllocate(bytes);
+    b.provided = b.mem != nullptr;
+  }
+  if (b.mem == nullptr) b.mem = std::aligned_alloc(64, bytes);
   if (b.mem == nullptr) fatalError(kFatalOther, "Failed to allocate RAM memory!");
   b.tag = 1;
   mBlocks.emplace(record.virtualAddress, b);
@@ -39,13 +50,17 @@ void RamLayer::deallocate(MemoryRecord record) {
   if (it == mBlocks.end()) return;
   if (it->second.locked)
     fatalError(kFatalBadAccess, "Double free on vaddr %zu", record.virtualAddress);
-  std::free(it->second.mem);
+  freeBlock(it->second);
   mBlocks.erase(it);
 }
 
 void RamLayer::lock(MemoryRecord record) {
   auto it = mBlocks.find(record.virtualAddress);
-  if (it != mBlocks.end()) it->second.locked = true;
+  if (it == mBlocks.end()) return;
+  it->second.locked = true;
+  // host code is about to touch the block: nothing the device still has queued
+  // out of it may be outstanding
+  if (it->second.provided && mQuiesce != nullptr) mQuiesce(it->second.mem);
 }
 
 void RamLayer::release(MemoryRecord record) {

@@ -58,13 +58,25 @@ public:
   size_t getTag(MemoryRecord record) override;
   void setTag(MemoryRecord record, size_t tag) override;
 
+  // blocks from a provider instead of the heap (see polar_rt_support_set_host_memory)
+  void setProvider(void* (*allocate)(size_t), void (*release)(void*), void (*quiesce)(void*)) {
+    mAllocate = allocate;
+    mRelease = release;
+    mQuiesce = quiesce;
+  }
+
 private:
   struct Block {
     void* mem = nullptr;
     size_t tag = 0;
     bool locked = false;
+    bool provided = false; // from the provider; heap otherwise
   };
+  void freeBlock(Block& b);
   std::unordered_map<size_t, Block> mBlocks;
+  void* (*mAllocate)(size_t) = nullptr;
+  void (*mRelease)(void*) = nullptr;
+  void (*mQuiesce)(void*) = nullptr;
 };
 
 class CoherentAllocator final : public BackendAllocator {
@@ -81,6 +93,10 @@ public:
   void release(const TensorInternal&) override;
 
   void registerDevice(Device& device) override;
+  // RAM-side blocks from a provider (polar_rt_support_set_host_memory)
+  void setHostMemory(void* (*allocate)(size_t), void (*release)(void*), void (*quiesce)(void*)) {
+    mRam->setProvider(allocate, release, quiesce);
+  }
   void allocate(const TensorInternal&, Device&) override;
   void allocate(const MemoryRecord& record, Device& device) override;
   void allocate(const MemoryRecord& record) override;
@@ -119,7 +135,7 @@ private:
   void refreshHost(const MemoryRecord& record);
 
   std::mutex mMutex;
-  std::unique_ptr<AllocatorLayerBase> mRam;
+  std::unique_ptr<RamLayer> mRam;
   std::vector<Slot> mSlots;
   std::unordered_map<size_t, State> mState; // by virtual address
 };

@@ -172,6 +172,16 @@ int polar_harness_device_kind(polar_harness* h) {
   return h ? static_cast<int>(h->inner->getKind()) : -1;
 }
 
+int polar_harness_use_plugin_host_memory(polar_harness* h) {
+  if (h == nullptr || h->lib == nullptr) return -1;
+  auto allocate = reinterpret_cast<void* (*)(size_t)>(dlsym(h->lib, "polarHostMemoryAllocate"));
+  auto release = reinterpret_cast<void (*)(void*)>(dlsym(h->lib, "polarHostMemoryRelease"));
+  auto quiesce = reinterpret_cast<void (*)(void*)>(dlsym(h->lib, "polarHostMemoryQuiesce"));
+  if (allocate == nullptr || release == nullptr || quiesce == nullptr) return -1;
+  h->allocator->setHostMemory(allocate, release, quiesce);
+  return 0;
+}
+
 uint64_t polar_harness_tensor(polar_harness* h, uint64_t dims, const uint64_t* shape) {
   if (h == nullptr || (dims > 0 && shape == nullptr)) return 0;
   TensorDecl t;

@@ -19,6 +19,13 @@ void polar_rt_support_register_device(BackendAllocator* allocator, Device* devic
   allocator->registerDevice(*device);
 }
 
+void polar_rt_support_set_host_memory(BackendAllocator* allocator, const polar_rt_host_memory* hooks) {
+  if (allocator == nullptr) fatalError(kFatalOther, "polar_rt_support_set_host_memory: null allocator");
+  auto* mine = static_cast<CoherentAllocator*>(allocator); // created by polar_rt_support_allocator_create
+  if (hooks == nullptr) mine->setHostMemory(nullptr, nullptr, nullptr);
+  else mine->setHostMemory(hooks->allocate, hooks->release, hooks->quiesce);
+}
+
 Device* polar_rt_support_host_device_create() {
   Device* host = new HostDevice();
   rememberDevice(*host, true);

@@ -221,6 +221,19 @@ void HipDevice::consumeEvent(Event* evt) {
   mIdleEvents.push_back(mine);
 }
 
+namespace {
+// Device through which polarHostMemoryAllocate takes pinned memory: the first
+// device of the most recently created context, null when there is none.
+std::mutex gHostMemoryMu;
+HipDevice* gHostMemoryDevice = nullptr;
+} // namespace
+
+HipContext::~HipContext() {
+  std::lock_guard<std::mutex> g(gHostMemoryMu);
+  for (auto& d : mDevices)
+    if (d.get() == gHostMemoryDevice) gHostMemoryDevice = nullptr;
+}
+
 HipContext::HipContext() {
   int n = 0;
   checkStatus(polar_hip_device_count(&n), "polar_hip_device_count");
@@ -233,6 +246,10 @@ HipContext::HipContext() {
     polar_hip_device_close(probe);
     mDevices.push_back(std::make_shared<HipDevice>(i));
   }
+  if (!mDevices.empty()) {
+    std::lock_guard<std::mutex> g(gHostMemoryMu);
+    gHostMemoryDevice = static_cast<HipDevice*>(mDevices.front().get());
+  }
 }
 
 } // namespace polarai::backend::generic::mi355x
@@ -244,6 +261,29 @@ polarai::backend::generic::Context* initContext() {
 }
 
 void closeContext(polarai::backend::generic::Context* ctx) { delete ctx; }
+
+// Optional extension, not part of the framework's interface: host memory for
+// the caller's RAM-side copies of tensors (the framework's TrivialAllocator
+// uses new[]: src/backend/generic/lib/allocators/TrivialAllocator.hpp:23-93).
+// Blocks from here are pinned; copyToDevice / copyToHost move bytes directly
+// between them and device memory instead of staging them.  Because an upload
+// out of such a block is only queued when copyToDevice returns, the caller calls
+// polarHostMemoryQuiesce(block) before the host writes the block again.
+// polarHostMemoryAllocate returns null when no context with a device exists.
+void* polarHostMemoryAllocate(size_t bytes) {
+  using namespace polarai::backend::generic::mi355x;
+  std::lock_guard<std::mutex> g(gHostMemoryMu);
+  if (gHostMemoryDevice == nullptr) return nullptr;
+  void* p = nullptr;
+  checkStatus(polar_hip_host_alloc(gHostMemoryDevice->native(), bytes, &p), "polar_hip_host_alloc");
+  return p;
+}
+void polarHostMemoryRelease(void* block) {
+  polarai::backend::generic::mi355x::checkStatus(polar_hip_host_free(block), "polar_hip_host_free");
+}
+void polarHostMemoryQuiesce(void* block) {
+  polarai::backend::generic::mi355x::checkStatus(polar_hip_host_quiesce(block), "polar_hip_host_quiesce");
+}
 
 }
 

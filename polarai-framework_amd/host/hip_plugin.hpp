@@ -125,7 +125,7 @@ private:
 class HipContext final : public Context {
 public:
   HipContext();
-  ~HipContext() override = default;
+  ~HipContext() override;
   std::vector<std::shared_ptr<Device>>& getDevices() override {
     return mDevices;
   }
