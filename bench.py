@@ -633,76 +633,85 @@ def bench_graphs():
     bias = np.zeros((256, 10), dtype=np.float32)
     y = (rng.random((256, 10)) < 0.1).astype(np.float32)
     g, _ = graphs.logreg_forward(x, w, bias, y)
-    with harness.Harness(plugin=LIB_PLUGIN) as h:
-        graphs.emit(g, h, {})
+
+    def evaluate(h, n=50):
         for _ in range(5):
             h.run()
         c0 = h.counters()
         ts = []
-        for _ in range(50):
+        for _ in range(n):
             t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
         c = h.counters()
-        phases = {name: round((getattr(c, "ns_" + name) - getattr(c0, "ns_" + name)) / 50 / 1e3, 1)
+        # host wall time per evaluation, mean of the n: the input nodes' host-side loads; per compute
+        # node allocate + lock (uploads happen here), the launch call, the releases; the barriers
+        phases = {name: round((getattr(c, "ns_" + name) - getattr(c0, "ns_" + name)) / n / 1e3, 1)
                   for name in ("input_nodes", "allocate_and_lock", "launch", "release", "barrier")}
-        out["logreg_forward"] = {
-            "workload": "X[256x784] W[784x10]: 4 input nodes, fmatmul_f_f -> fadd -> fsigmoid -> flogloss, "
-                        "one barrier per cluster, inputs re-loaded every evaluation as the framework does",
-            "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
-            "mean_us": round(float(np.mean(ts)) * 1e6, 1),
-            "phase_us": phases,  # host wall time per evaluation, mean of the 50: the input nodes' host-side
-                                 # loads; per compute node allocate + lock (uploads happen here), the
-                                 # launch call, the releases; the barriers after the clusters
-            "launches_per_evaluate": 4,
-            "uploads_per_evaluate": int((c.copies_to_device - c0.copies_to_device) // 50),
-            "upload_bytes_per_evaluate": int((c.bytes_to_device - c0.bytes_to_device) // 50)}
-        log(f"  phases (us): {phases}")
-        log(f"logreg forward through the plugin: {out['logreg_forward']['evaluate_us']} us per evaluation")
-    # the same forward pass with the extended (fused) builtins: 2 launches instead of 4
-    with harness.Harness(plugin=LIB_PLUGIN) as h:
+        return {"evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
+                "mean_us": round(float(np.mean(ts)) * 1e6, 1), "phase_us": phases,
+                "uploads_per_evaluate": int((c.copies_to_device - c0.copies_to_device) // n),
+                "upload_bytes_per_evaluate": int((c.bytes_to_device - c0.bytes_to_device) // n)}
+
+    def fused(h):
         X, W, B, Y = h.input(x), h.input(w), h.input(bias), h.input(y)
         h.end_cluster()
         p = h.fmatmul_fadd_fsigmoid(False, False, X, W, 1.0, B, 1.0)
         h.end_cluster()
         # flogloss consumes the sigmoid; the fused sigmoid+logloss would need the pre-activation,
         # which the first fused launch does not keep
-        loss = h.flogloss(p, Y)
+        h.flogloss(p, Y)
         h.end_cluster()
-        for _ in range(5):
-            h.run()
-        ts = []
-        for _ in range(50):
-            t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
-        out["logreg_forward_fused"] = {
-            "workload": "same inputs; fmatmul_f_f_fadd_fsigmoid -> flogloss (extended builtins)",
-            "evaluate_us": round(float(np.median(ts)) * 1e6, 1), "min_us": round(float(np.min(ts)) * 1e6, 1),
-            "launches_per_evaluate": 2}
-        log(f"logreg forward, fused builtins: {out['logreg_forward_fused']['evaluate_us']} us per evaluation")
+
+    for key, pinned in (("logreg_forward", False), ("logreg_forward_plugin_ram", True)):
+        with harness.Harness(plugin=LIB_PLUGIN, plugin_host_memory=pinned) as h:
+            graphs.emit(g, h, {})
+            r = evaluate(h)
+        r["workload"] = ("X[256x784] W[784x10]: 4 input nodes, fmatmul_f_f -> fadd -> fsigmoid -> flogloss, "
+                         "one barrier per cluster, inputs re-loaded every evaluation as the framework does; "
+                         + ("the caller's RAM-side blocks in the plugin's pinned host memory (optional "
+                            "polarHostMemory* symbols): uploads are not staged" if pinned else
+                            "the caller's RAM-side blocks on the heap, as the framework's allocator keeps them"))
+        r["launches_per_evaluate"] = 4
+        out[key] = r
+        log(f"  phases (us): {r['phase_us']}")
+        log(f"{key} through the plugin: {r['evaluate_us']} us per evaluation")
+    # the same forward pass with the extended (fused) builtins: 2 launches instead of 4
+    for key, pinned in (("logreg_forward_fused", False), ("logreg_forward_fused_plugin_ram", True)):
+        with harness.Harness(plugin=LIB_PLUGIN, plugin_host_memory=pinned) as h:
+            fused(h)
+            r = evaluate(h)
+        r["workload"] = ("same inputs; fmatmul_f_f_fadd_fsigmoid -> flogloss (extended builtins)"
+                         + ("; RAM-side blocks in the plugin's pinned host memory" if pinned else ""))
+        r["launches_per_evaluate"] = 2
+        out[key] = r
+        log(f"{key}: {r['evaluate_us']} us per evaluation")
     rng = np.random.default_rng(71)
     x = rng.random((1024, 1024), dtype=np.float32)
     w1 = (rng.standard_normal((1024, 4096)) / 32).astype(np.float32)
     w2 = (rng.standard_normal((4096, 1024)) / 64).astype(np.float32)
     y = (rng.random((1024, 1024)) < 0.5).astype(np.float32)
     f, gr, u, _ = graphs.mlp_graphs(x, w1, w2, y)
-    with harness.Harness(plugin=LIB_PLUGIN) as h:
-        tensors = {}
-        times = {}
-        for graph in (f, gr, u):
-            graphs.emit(graph, h, tensors)
-            h.run()  # first evaluation allocates
-            ts = []
-            for _ in range(3):
-                t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
-            times[graph.name] = float(np.median(ts))
-            h.clear_program()
-        out["mlp_forward_backward"] = {
-            "workload": "batch 1024, 1024->4096->1024, sigmoid, logloss; forward, the framework's gradient "
-                        "graph and its in-place weight update, each evaluated through the plugin",
-            "forward_ms": round(times["mlp_forward"] * 1e3, 3),
-            "gradient_ms": round(times["mlp_gradient"] * 1e3, 3),
-            "update_ms": round(times["mlp_update"] * 1e3, 3),
-            "nodes": {gph.name: len(gph.nodes) for gph in (f, gr, u)}}
-        log(f"mlp through the plugin: forward {times['mlp_forward'] * 1e3:.2f} ms, gradient "
-            f"{times['mlp_gradient'] * 1e3:.2f} ms, update {times['mlp_update'] * 1e3:.2f} ms")
+    for key, pinned in (("mlp_forward_backward", False), ("mlp_forward_backward_plugin_ram", True)):
+        with harness.Harness(plugin=LIB_PLUGIN, plugin_host_memory=pinned) as h:
+            tensors = {}
+            times = {}
+            for graph in (f, gr, u):
+                graphs.emit(graph, h, tensors)
+                h.run()  # first evaluation allocates
+                ts = []
+                for _ in range(3):
+                    t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
+                times[graph.name] = float(np.median(ts))
+                h.clear_program()
+            out[key] = {
+                "workload": "batch 1024, 1024->4096->1024, sigmoid, logloss; forward, the framework's gradient "
+                            "graph and its in-place weight update, each evaluated through the plugin"
+                            + ("; RAM-side blocks in the plugin's pinned host memory" if pinned else ""),
+                "forward_ms": round(times["mlp_forward"] * 1e3, 3),
+                "gradient_ms": round(times["mlp_gradient"] * 1e3, 3),
+                "update_ms": round(times["mlp_update"] * 1e3, 3),
+                "nodes": {gph.name: len(gph.nodes) for gph in (f, gr, u)}}
+            log(f"{key}: forward {times['mlp_forward'] * 1e3:.2f} ms, gradient "
+                f"{times['mlp_gradient'] * 1e3:.2f} ms, update {times['mlp_update'] * 1e3:.2f} ms")
     return out
 
 

@@ -5,6 +5,7 @@
 #include "polar_harness.h"
 #include "polar_rt_support.hpp"
 #include "devices.hpp"
+#include "coherent_allocator.hpp"
 
 #include <cstdio>
 #include <cstdlib>
@@ -59,8 +60,70 @@ static void evictionScanSurvivesMutatingCallback() {
   CHECK(layer.isAllocated(MemoryRecord{1000, 64}));
 }
 
+// RAM-side blocks taken from a provider (polar_rt_support_set_host_memory): the
+// provider is asked once per record, a null answer falls back to the heap,
+// quiesce runs before every host access to a provided block and never for a
+// heap one, and every provided block goes back through release.
+namespace provider {
+int allocated = 0, released = 0, quiesced = 0, refused = 0;
+void* lastQuiesced = nullptr;
+void* allocate(size_t bytes) {
+  if (bytes > 4096) {
+    ++refused;
+    return nullptr;
+  }
+  ++allocated;
+  return std::malloc(bytes);
+}
+void release(void* p) {
+  ++released;
+  std::free(p);
+}
+void quiesce(void* p) {
+  ++quiesced;
+  lastQuiesced = p;
+}
+} // namespace provider
+
+static void ramBlocksFromAProvider() {
+  using polarai::backend::generic::MemoryRecord;
+  using LockType = polarai::core::internal::LockType;
+  auto* allocator = polar_rt_support_allocator_create();
+  auto* host = polar_rt_support_host_device_create();
+  const polar_rt_host_memory hooks{provider::allocate, provider::release, provider::quiesce};
+  polar_rt_support_set_host_memory(allocator, &hooks);
+  polar_rt_support_register_device(allocator, host);
+  const MemoryRecord small{1, 256}, other{1000, 512}, big{5000, 1 << 20};
+  allocator->allocate(small);
+  allocator->allocate(other);
+  allocator->allocate(big); // the provider refuses it: heap
+  CHECK(provider::allocated == 2 && provider::refused == 1);
+  allocator->allocate(small); // already there: the provider is not asked again
+  CHECK(provider::allocated == 2);
+  CHECK(provider::quiesced == 0);
+  allocator->lock(small, *host, LockType::READ_WRITE);
+  CHECK(provider::quiesced == 1);
+  auto* p = allocator->get<float>(small, *host);
+  CHECK(p != nullptr && provider::lastQuiesced == static_cast<void*>(p));
+  for (int i = 0; i < 64; ++i) p[i] = float(i);
+  allocator->release(small, *host);
+  allocator->lock(big, *host, LockType::READ_WRITE);
+  CHECK(provider::quiesced == 1); // heap block: nothing to wait for
+  allocator->get<float>(big, *host)[(1 << 18) - 1] = 1.0f;
+  allocator->release(big, *host);
+  allocator->lock(small, *host, LockType::READ);
+  CHECK(provider::quiesced == 2 && allocator->get<float>(small, *host)[63] == 63.0f);
+  allocator->release(small, *host);
+  static_cast<polar_harness_detail::CoherentAllocator*>(allocator)->deallocate(small);
+  CHECK(provider::released == 1);
+  polar_rt_support_host_device_destroy(host);
+  polar_rt_support_allocator_destroy(allocator); // gives back what is left
+  CHECK(provider::released == 2);
+}
+
 int main() {
   evictionScanSurvivesMutatingCallback();
+  ramBlocksFromAProvider();
   for (int round = 0; round < 3; ++round) {
     polar_harness* h = nullptr;
     CHECK(polar_harness_open(nullptr, 0, &h) == 0);

@@ -2,6 +2,8 @@
 (include/polar_hip.h).  Bit-exact for the operations that are single IEEE
 operations or pure data movement; 1e-5 relative per element for
 sigmoid/logloss; 1e-4 relative Frobenius for matmul."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -415,6 +417,63 @@ def test_copy_to_device_of_large_buffers_round_trips(dev, nbytes):
     src[:] = -1.0                      # the call has taken its copy
     assert np.array_equal(d.download(), keep)
     d.free()
+
+
+@pytest.mark.parametrize("nbytes", [20, 4096 + 4, 3 * 1024 * 1024, 8 * 1024 * 1024, 9 * 1024 * 1024 + 12])
+def test_copies_through_pinned_host_blocks(dev, nbytes):
+    """A block of polar_hip_host_alloc is moved directly: an upload is queued when the call
+    returns (quiesce before rewriting the block), a read-back is complete."""
+    _say("host block", nbytes)
+    count = nbytes // 4
+    block = dev.host_alloc(nbytes + 64)
+    try:
+        host = np.ctypeslib.as_array(C.cast(block, C.POINTER(C.c_float)), shape=(count + 16,))
+        d = dev.empty(count)
+        for step in range(3):
+            dev.host_quiesce(block)
+            host[:count] = (np.arange(count, dtype=np.int64) % 16000057 + step).astype(np.float32)
+            expect = host[:count].copy()
+            dev.copy_to_device(d.ptr, block, nbytes)
+            assert np.array_equal(d.download(), expect)          # pageable destination: staged
+            dev.host_quiesce(block + 8)                            # any address inside the block
+            host[:] = -1.0
+            dev.copy_to_host(block + 16, d.ptr, nbytes)            # into the block, off its base
+            assert np.array_equal(host[4:4 + count], expect)
+            assert host[4 + count] == -1.0 and host[3] == -1.0
+        d.free()
+    finally:
+        dev.host_free(block)
+
+
+def test_pinned_host_block_calls_reject_foreign_pointers(dev):
+    buf = np.zeros(16, dtype=np.float32)
+    with pytest.raises(Exception):
+        dev.host_free(buf.ctypes.data)
+    with pytest.raises(Exception):
+        dev.host_quiesce(buf.ctypes.data)
+    dev.host_free(None)
+    dev.host_quiesce(None)
+
+
+@pytest.mark.parametrize("count", [5000, 150000, 262144])
+def test_many_small_uploads_without_a_wait_between(dev, count):
+    """More one- and two-slot uploads than the staging ring has slots, with no wait in between:
+    a slot is only reused once the transfer out of it is over."""
+    _say("small uploads", count)
+    rng = np.random.default_rng(count)
+    src = np.empty(count, dtype=np.float32)
+    targets, expect = [], []
+    for i in range(40):
+        src[:] = rng.random(count, dtype=np.float32) + i
+        expect.append(src.copy())
+        d = dev.empty(count)
+        dev.copy_to_device(d.ptr, src.ctypes.data, count * 4)
+        targets.append(d)
+        if i == 20:
+            dev.record().synchronize()       # tells the library how far the stream has got
+    for i, d in enumerate(targets):
+        assert np.array_equal(d.download(), expect[i]), i
+        d.free()
 
 
 def test_pool_reuses_blocks(dev):

@@ -21,9 +21,12 @@ def _say(*a):
     print(*a, flush=True)
 
 
-@pytest.fixture()
-def h():
-    hh = harness.Harness(plugin=LIB_PLUGIN)  # raises if no MI355X is found
+@pytest.fixture(params=["heap_ram", "plugin_ram"])
+def h(request):
+    """The caller's RAM-side blocks on the heap (as the framework's allocator keeps them) and in
+    the plugin's pinned host memory (its optional polarHostMemory* symbols)."""
+    hh = harness.Harness(plugin=LIB_PLUGIN,  # raises if no MI355X is found
+                         plugin_host_memory=request.param == "plugin_ram")
     yield hh
     hh.close()
 
@@ -135,6 +138,25 @@ def test_coherence_counts_on_gpu(h):
     assert k["events_waited"] == 2 and k["deferred_releases"] == 6
     assert np.array_equal(h.read(d), (np.arange(1024, dtype=np.float32) + 1) * np.arange(1024, dtype=np.float32))
     assert _counters(h)["copies_to_host"] == 1
+
+
+def test_rewritten_ram_block_reaches_the_device(h):
+    """Host code rewrites a tensor between evaluations: every evaluation sees the new values, also
+    when the upload out of the RAM block was only queued when the previous evaluation returned."""
+    n = 3 << 16
+    a = h.tensor(n)
+    h.holder(a)
+    h.end_cluster()
+    c = h.fadd(a, 1.0, a, 2.0)
+    h.end_cluster()
+    for i in range(6):
+        data = np.arange(n, dtype=np.float32) % 977 + i
+        h.host_write(a, data)
+        h.run()
+        if i % 2:                          # read back on some evaluations, rewrite at once on others
+            assert np.array_equal(h.read(c), data * 3), i
+    assert np.array_equal(h.read(c), data * 3)
+    assert np.array_equal(h.read(a), data)
 
 
 def test_logreg_forward_config(h):
