@@ -54,6 +54,21 @@ def test_plugin_exports_driver_entry_points():
     assert hasattr(lib, "initContext") and hasattr(lib, "closeContext")
 
 
+def test_plugin_exports_the_optional_host_memory_symbols():
+    lib = C.CDLL(LIB_PLUGIN, mode=os.RTLD_LAZY | os.RTLD_LOCAL)
+    for name in ("polarHostMemoryAllocate", "polarHostMemoryRelease", "polarHostMemoryQuiesce"):
+        assert hasattr(lib, name), name
+    # no context has been created in this process: there is no device to pin memory through
+    lib.polarHostMemoryAllocate.restype = C.c_void_p
+    lib.polarHostMemoryAllocate.argtypes = [C.c_size_t]
+    assert lib.polarHostMemoryAllocate(4096) is None
+
+
+def test_mock_device_has_no_plugin_host_memory():
+    with pytest.raises(RuntimeError):
+        harness.Harness(plugin=None, plugin_host_memory=True)
+
+
 def test_device_library_without_gpu_reports_no_device():
     if capi.device_count() != 0:
         pytest.skip("a GPU is present")
