@@ -253,6 +253,7 @@ def main():
         result["next_builtins"] = bench_next_builtins(dev, da, n, args)
         if not args.no_ragged:
             result["ragged"] = bench_ragged(dev, args)
+            result["matmul_mid_size"] = bench_matmul_mid(dev, args)
             result["copies"] = bench_copies(dev)
     da.free(); db.free()
     dev.close()
@@ -555,6 +556,39 @@ def bench_ragged(dev, args):
         log(f"fmatmul {label}: {t * 1e6:7.1f} us per call (first kernel {first * 1e6:.1f} us)  "
             f"{flops / t / 1e12:6.2f} TFLOP/s  {nbytes / t / 1e9:7.1f} GB/s of compulsory traffic")
         for x in (da, db, dc):
+            x.free()
+    return out
+
+
+def bench_matmul_mid(dev, args):
+    """Matmuls between the two extremes: the MLP configuration's products (batch 1024,
+    1024 -> 4096 -> 1024, forward and gradient graphs) and a few cubes.  Too short for the
+    clock to settle, so they are timed as a graph meets them: a handful of untimed calls,
+    then calls issued back to back over four sets of operands, events around each call
+    (a split contraction's reduction kernel included)."""
+    out = {"timing": "per call, issued back to back over 4 sets of operands, events around each call"}
+    rng = np.random.default_rng(12)
+    reps = max(20, args.steps)
+    sets = 4
+    for ta, tb, m, n, k in ((0, 0, 1024, 4096, 1024), (0, 0, 1024, 1024, 4096), (0, 1, 1024, 4096, 1024),
+                            (1, 0, 1024, 4096, 1024), (1, 0, 4096, 1024, 1024), (0, 0, 512, 512, 512),
+                            (0, 0, 1024, 1024, 1024), (0, 0, 2048, 2048, 2048), (0, 0, 3072, 3072, 3072)):
+        sa, sb = ((k, m) if ta else (m, k)), ((n, k) if tb else (k, n))
+        das = device_copies(dev, dev.array(rng.standard_normal(sa, dtype=np.float32)), m * k, sets)
+        dbs = device_copies(dev, dev.array(rng.standard_normal(sb, dtype=np.float32)), k * n, sets)
+        dcs = [dev.empty(m * n) for _ in range(sets)]
+        call = lambda i: dev.fmatmul(ta, tb, das[i % sets], dbs[i % sets], dcs[i % sets], m, n, k)
+        t = float(np.median(time_calls(dev, call, 6, reps))) * 1e-3
+        config, splits, tile = dev.fmatmul_plan(m, n, k)
+        flops = 2.0 * m * n * k
+        name = f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'} {m}x{n}x{k}"
+        out[name] = {"M": m, "N": n, "K": k, "us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1),
+                     "frac_mfma_fp32_peak": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+                     "tile": "x".join(map(str, tile)), "k_splits": splits}
+        log(f"{name:34s} {t * 1e6:8.1f} us  {flops / t / 1e12:6.1f} TFLOP/s  "
+            f"({flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS * 100:.0f} % of the fp32 matrix peak; "
+            f"tile {'x'.join(map(str, tile))}, {splits} k-split(s))")
+        for x in das + dbs + dcs:
             x.free()
     return out
 

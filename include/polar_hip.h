@@ -199,6 +199,23 @@ int polar_hip_ftranspose(polar_hip_device* dev, const float* in, float* out,
 int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
                       const float* a, const float* b, float* c, uint64_t m,
                       uint64_t n, uint64_t k);
+/* How polar_hip_fmatmul would compute an M x N x K product (no counterpart in
+ * the reference; for tuning and tests): the tile configuration its planner
+ * picks (an index into the library's table; -1 for the shapes taken by the
+ * short-contraction kernels), the number of parts the contraction is split
+ * into, and, if tile is not null, the tile's extent along M, N and K. */
+int polar_hip_fmatmul_plan(polar_hip_device* dev, uint64_t m, uint64_t n,
+                           uint64_t k, int* tile_config, uint32_t* splits,
+                           uint32_t tile[3]);
+#define POLAR_HIP_MATMUL_TILE_CONFIGS 10
+/* polar_hip_fmatmul with the tile configuration (0 .. POLAR_HIP_MATMUL_TILE_
+ * CONFIGS - 1) and split count (1 .. 256; reduced to what K can fill) given by
+ * the caller instead of the planner.  Same result up to the order of the
+ * additions along K. */
+int polar_hip_fmatmul_with_plan(polar_hip_device* dev, int transA, int transB,
+                                const float* a, const float* b, float* c,
+                                uint64_t m, uint64_t n, uint64_t k,
+                                int tile_config, uint32_t splits);
 
 /* ---- Code objects compiled elsewhere (the framework's JIT) --------------------
  * Counterpart of the module handling in the reference's CUDA runtime

@@ -86,6 +86,9 @@ SIGNATURES = {
     "polar_hip_ffill": (_i, [_vp, _f, _vp, _u64]),
     "polar_hip_ftranspose": (_i, [_vp, _vp, _vp, _u64, _u64]),
     "polar_hip_fmatmul": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
+    "polar_hip_fmatmul_plan": (_i, [_vp, _u64, _u64, _u64, C.POINTER(_i), C.POINTER(C.c_uint32),
+                                    C.POINTER(C.c_uint32)]),
+    "polar_hip_fmatmul_with_plan": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64, _i, C.c_uint32]),
     "polar_hip_module_load": (_i, [_vp, _vp, _u64, C.POINTER(_vp)]),
     "polar_hip_module_unload": (_i, [_vp, _vp]),
     "polar_hip_module_has_kernel": (_i, [_vp, C.c_char_p, C.POINTER(_i)]),
@@ -340,6 +343,16 @@ class Device:
     def fsigmoid_flogloss(self, x, truth, out, n=None):
         _check(self.lib, self.lib.polar_hip_fsigmoid_flogloss(self.handle, x.ptr, truth.ptr, out.ptr,
                                                               out.count if n is None else n))
+
+    def fmatmul_plan(self, m, n, k):
+        """(tile configuration or -1, splits, (tile M, tile N, tile K)) the planner picks."""
+        cfg, splits, tile = _i(0), C.c_uint32(0), (C.c_uint32 * 3)()
+        _check(self.lib, self.lib.polar_hip_fmatmul_plan(self.handle, m, n, k, C.byref(cfg), C.byref(splits), tile))
+        return cfg.value, splits.value, tuple(tile)
+
+    def fmatmul_with_plan(self, trans_a, trans_b, a, b, c, m, n, k, tile_config, splits):
+        _check(self.lib, self.lib.polar_hip_fmatmul_with_plan(
+            self.handle, int(bool(trans_a)), int(bool(trans_b)), a.ptr, b.ptr, c.ptr, m, n, k, tile_config, splits))
 
     def fmatmul(self, trans_a, trans_b, a, b, c, m, n, k):
         _check(self.lib, self.lib.polar_hip_fmatmul(

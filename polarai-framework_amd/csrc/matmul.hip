@@ -12,7 +12,9 @@
 //   * operand contiguous along x (A transposed, B not transposed): a lane
 //     loads 4 consecutive x of one k and stores them as one 16-byte LDS write.
 // The next tile is fetched into registers while the current one is multiplied
-// (two LDS stages, one barrier per step).  Each wave owns a (BM/WM) x (BN/WN)
+// (two LDS stages, one barrier per step); tiles smaller than 256 x 256 fetch two
+// steps ahead, because one of their k-steps (0.8-2.6 us) is shorter than a
+// trip to memory.  Each wave owns a (BM/WM) x (BN/WN)
 // sub-tile as TM x TN accumulator blocks of 32x32; per k-pair it reads TM + TN
 // LDS words per lane and issues TM*TN MFMAs.  The LDS row pitch is chosen per
 // operand so that neither the fill nor the fragment reads collide on banks.
@@ -39,11 +41,13 @@
 // K) are split along K: every split writes its partial product to a workspace
 // from the device pool and a second kernel adds the partials in split order,
 // so the result does not depend on scheduling.  Tile shape and split count
-// come from a small cost model (planMatmul) of rounds x k-steps x step time.
+// come from a small cost model (planMatmul) of rounds x k-steps x step time,
+// with step times measured per tile shape on the full chip.
 #include "internal.h"
 #include "matmul_epilogue.h"
 
 #include <cmath>
+#include <type_traits>
 
 
 using namespace polar_hip_detail;
@@ -183,9 +187,13 @@ __device__ __forceinline__ void tileOfGroup(uint32_t bid, uint32_t nGroups,
   tn = in / rows;
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB, bool VEC,
+// PF = how many k-steps ahead operand tiles are fetched into registers: 1 (the
+// tile of step kt + 1 travels while step kt is multiplied) or 2 (two tiles in
+// flight, for small tiles whose k-step is shorter than the memory latency).
+template <int BM, int BN, int BK, int WM, int WN, int PF, bool TA, bool TB, bool VEC,
           bool EDGE>
 __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
+  static_assert(PF == 1 || PF == 2, "prefetch distance");
   constexpr int NT = WM * WN * 64;
   constexpr int WTM = BM / WM, WTN = BN / WN;
   constexpr int TM = WTM / 32, TN = WTN / 32;
@@ -212,8 +220,8 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
 
   // A: k-contiguous when not transposed ([M x K]); B: k-contiguous when
   // transposed ([N x K]).
-  TileFetch<BM, BK, NT, !TA, VEC, EDGE> fa;
-  TileFetch<BN, BK, NT, TB, VEC, EDGE> fb;
+  TileFetch<BM, BK, NT, !TA, VEC, EDGE> fa[PF];
+  TileFetch<BN, BK, NT, TB, VEC, EDGE> fb[PF];
   const size_t lda = TA ? p.M : p.K;
   const size_t ldb = TB ? p.K : p.N;
 
@@ -227,10 +235,14 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
 
   const uint32_t nk = kEnd > kBegin ? (kEnd - kBegin + BK - 1) / BK : 0;
   if (nk != 0) { // uniform; the host never creates an empty split
-    fa.load(p.A, lda, m0, kBegin, p.M, kEnd, t);
-    fb.load(p.B, ldb, n0, kBegin, p.N, kEnd, t);
-    fa.store(As[0], t);
-    fb.store(Bs[0], t);
+    fa[0].load(p.A, lda, m0, kBegin, p.M, kEnd, t);
+    fb[0].load(p.B, ldb, n0, kBegin, p.N, kEnd, t);
+    fa[0].store(As[0], t);
+    fb[0].store(Bs[0], t);
+    if (PF == 2 && nk > 1) { // the tile of step 1 stays in registers until step 0 ends
+      fa[0].load(p.A, lda, m0, kBegin + BK, p.M, kEnd, t);
+      fb[0].load(p.B, ldb, n0, kBegin + BK, p.N, kEnd, t);
+    }
   }
   __syncthreads();
 
@@ -238,34 +250,76 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
   const int bBase = wn * WTN + (lane % 32);
   const int kLane = lane / 32;
 
-  for (uint32_t kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    const bool more = kt + 1 < nk;
-    if (more) {
-      fa.load(p.A, lda, m0, kBegin + (kt + 1) * BK, p.M, kEnd, t);
-      fb.load(p.B, ldb, n0, kBegin + (kt + 1) * BK, p.N, kEnd, t);
+  if constexpr (PF == 1) {
+    for (uint32_t kt = 0; kt < nk; ++kt) {
+      const int cur = kt & 1;
+      const bool more = kt + 1 < nk;
+      if (more) {
+        fa[0].load(p.A, lda, m0, kBegin + (kt + 1) * BK, p.M, kEnd, t);
+        fb[0].load(p.B, ldb, n0, kBegin + (kt + 1) * BK, p.N, kEnd, t);
+      }
+      const float* as = As[cur];
+      const float* bs = Bs[cur];
+#pragma unroll
+      for (int kk = 0; kk < BK; kk += 2) {
+        float a[TM], b[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a[i] = as[(kk + kLane) * LDA + aBase + i * 32];
+#pragma unroll
+        for (int j = 0; j < TN; ++j) b[j] = bs[(kk + kLane) * LDB + bBase + j * 32];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j],
+                                                            0, 0, 0);
+      }
+      if (more) {
+        fa[0].store(As[cur ^ 1], t);
+        fb[0].store(Bs[cur ^ 1], t);
+      }
+      __syncthreads();
     }
-    const float* as = As[cur];
-    const float* bs = Bs[cur];
+  } else {
+    // One k-step: fetch the tile two steps ahead into register set `into`,
+    // multiply the LDS stage of step kt, then move the tile of step kt + 1
+    // (register set `from`) into the other stage.
+    auto step = [&](uint32_t kt, auto fromTag, auto intoTag) {
+      constexpr int from = decltype(fromTag)::value, into = decltype(intoTag)::value;
+      const int cur = kt & 1;
+      if (kt + 2 < nk) {
+        fa[into].load(p.A, lda, m0, kBegin + (kt + 2) * BK, p.M, kEnd, t);
+        fb[into].load(p.B, ldb, n0, kBegin + (kt + 2) * BK, p.N, kEnd, t);
+      }
+      const float* as = As[cur];
+      const float* bs = Bs[cur];
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float a[TM], b[TN];
+      for (int kk = 0; kk < BK; kk += 2) {
+        float a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a[i] = as[(kk + kLane) * LDA + aBase + i * 32];
+        for (int i = 0; i < TM; ++i) a[i] = as[(kk + kLane) * LDA + aBase + i * 32];
 #pragma unroll
-      for (int j = 0; j < TN; ++j) b[j] = bs[(kk + kLane) * LDB + bBase + j * 32];
+        for (int j = 0; j < TN; ++j) b[j] = bs[(kk + kLane) * LDB + bBase + j * 32];
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j],
-                                                          0, 0, 0);
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j],
+                                                            0, 0, 0);
+      }
+      if (kt + 1 < nk) {
+        fa[from].store(As[cur ^ 1], t);
+        fb[from].store(Bs[cur ^ 1], t);
+      }
+      __syncthreads();
+    };
+    // at the start of step kt register set kt % 2 holds the tile of step kt + 1
+    using Set0 = std::integral_constant<int, 0>;
+    using Set1 = std::integral_constant<int, PF - 1>;
+    for (uint32_t kt = 0; kt < nk; kt += 2) {
+      step(kt, Set0{}, Set1{});
+      if (kt + 1 < nk) step(kt + 1, Set1{}, Set0{});
     }
-    if (more) {
-      fa.store(As[cur ^ 1], t);
-      fb.store(Bs[cur ^ 1], t);
-    }
-    __syncthreads();
   }
 
   // Accumulator block layout of the 32x32 MFMA: register r of lane l holds
@@ -343,23 +397,23 @@ hipError_t launchReduce(polar_hip_device* dev, const float* partial, float* c, u
                       p.epilogue, p.bias, p.scaleAcc, p.scaleBias);
 }
 
-template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
+template <int BM, int BN, int BK, int WM, int WN, int PF, bool TA, bool TB>
 int launchLayout(polar_hip_device* dev, const MatmulArgs& p, bool vec, bool edge) {
   const uint64_t groups = uint64_t(p.tilesM) * p.tilesN * p.kSplits;
   const dim3 grid(static_cast<unsigned>(groups)), block(WM * WN * 64);
   if (vec && !edge)
     POLAR_HIP_TRY(launchKernel(
-        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, false>, grid, block, p));
+        dev, matmulKernel<BM, BN, BK, WM, WN, PF, TA, TB, true, false>, grid, block, p));
   else if (vec && edge)
     POLAR_HIP_TRY(launchKernel(
-        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, true, true>, grid, block, p));
+        dev, matmulKernel<BM, BN, BK, WM, WN, PF, TA, TB, true, true>, grid, block, p));
   else
     POLAR_HIP_TRY(launchKernel(
-        dev, matmulKernel<BM, BN, BK, WM, WN, TA, TB, false, true>, grid, block, p));
+        dev, matmulKernel<BM, BN, BK, WM, WN, 1, TA, TB, false, true>, grid, block, p));
   return POLAR_HIP_OK;
 }
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, int PF = 1>
 int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
                uint32_t splits) {
   MatmulArgs p = p0;
@@ -395,10 +449,10 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
     p.C = static_cast<float*>(workspace);
   }
   int st;
-  if (!ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, false, false>(dev, p, vec, edge);
-  else if (!ta && tb) st = launchLayout<BM, BN, BK, WM, WN, false, true>(dev, p, vec, edge);
-  else if (ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, true, false>(dev, p, vec, edge);
-  else st = launchLayout<BM, BN, BK, WM, WN, true, true>(dev, p, vec, edge);
+  if (!ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, PF, false, false>(dev, p, vec, edge);
+  else if (!ta && tb) st = launchLayout<BM, BN, BK, WM, WN, PF, false, true>(dev, p, vec, edge);
+  else if (ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, PF, true, false>(dev, p, vec, edge);
+  else st = launchLayout<BM, BN, BK, WM, WN, PF, true, true>(dev, p, vec, edge);
   if (splits > 1 && st == POLAR_HIP_OK) {
     hipError_t e = launchReduce(dev, static_cast<const float*>(workspace), c, count, splits, p);
     if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
@@ -408,17 +462,26 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
 
 // ---- tile shape and split count -----------------------------------------------
 struct TileConfig {
-  int bm, bn, bk, waves, residentGroups;
-  float mfmaEfficiency; // fraction of the matrix pipe a lone group can use
+  int bm, bn, bk;
+  int residentGroups; // groups of this shape one CU holds (LDS, lanes)
+  // Microseconds per k-step, measured with every CU busy (cold clock, as a lone
+  // launch in a graph finds it): stepAlone with one group on the CU, and what
+  // every co-resident group adds once the groups no longer hide in each other's
+  // latency; a step with r groups resident takes max(stepAlone, r * stepPerGroup).
+  float stepAlone, stepPerGroup;
 };
-// order = the switch in polar_hip_fmatmul
+// order = the switch in matmulWithEpilogue
 constexpr TileConfig kConfigs[] = {
-    {256, 256, 32, 16, 1, 0.92f}, // 4x4 waves of 64x64: one group per CU
-    {128, 128, 16, 4, 2, 0.85f},  // 2x2 waves of 64x64
-    {64, 64, 16, 4, 4, 0.60f},   // 2x2 waves of 32x32
-    {128, 32, 32, 4, 2, 0.55f},  // skinny N
-    {32, 128, 32, 4, 2, 0.55f},  // skinny M
-    {32, 32, 32, 1, 8, 0.15f},   // one wave
+    {256, 256, 32, 1, 8.2f, 8.2f},   // 4x4 waves of 64x64: one group per CU; 7.8 warm, 8.4-9.0 cold
+    {128, 128, 32, 2, 2.6f, 2.28f},  // 2x4 waves of 64x32, tiles fetched two steps ahead
+    {64, 64, 32, 4, 0.79f, 0.74f},   // 2x2 waves of 32x32, two steps ahead
+    {128, 32, 32, 3, 0.85f, 0.77f},  // skinny N
+    {32, 128, 32, 3, 0.85f, 0.77f},  // skinny M
+    {32, 32, 32, 8, 1.0f, 0.22f},    // one wave (0.78 in a long loop; short loops measured 10 % behind the others)
+    {256, 128, 32, 1, 4.65f, 4.65f}, // 4x2 waves of 64x64, two steps ahead
+    {128, 256, 32, 1, 4.6f, 4.6f},   // 2x4 waves of 64x64, two steps ahead
+    {128, 64, 32, 3, 1.32f, 1.38f},  // 4x2 waves of 32x32, two steps ahead
+    {64, 128, 32, 3, 1.32f, 1.38f},  // 2x4 waves of 32x32, two steps ahead
 };
 
 struct MatmulPlan {
@@ -426,10 +489,13 @@ struct MatmulPlan {
   uint32_t splits;
 };
 
-// Estimated microseconds = rounds x k-steps x step time (+ reduction).  A step
-// of a lone group is bound by the latency of its global->LDS->MFMA chain
-// (about 1.3 us, measured); co-resident groups overlap until they saturate the
-// CU's matrix pipe (256 flop/clk at 2.4 GHz).
+// Estimated microseconds of every tile shape and split count; the cheapest
+// wins.  The groups run in rounds of (CUs x resident groups); a k-step of a
+// round costs what the table says for the number of groups a CU holds in it,
+// and a partly filled last round takes as long per step as its fullest CU
+// (4097^3 on 256x256 tiles is 289 groups = 2 rounds, not 1.13).  On top: launch,
+// filling the pipeline and storing C (a few steps' worth), and for split
+// contractions the second kernel that adds the partial products.
 MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
   static const uint32_t kSplitChoices[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128, 192, 256};
   MatmulPlan best{1, 1};
@@ -438,18 +504,19 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
     const TileConfig& t = kConfigs[c];
     const double tiles = double((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
     const uint32_t kSteps = (k + t.bk - 1) / t.bk;
-    const double mfmaUs = 2.0 * t.bm * t.bn * t.bk / (256.0 * 2400.0 * t.mfmaEfficiency);
+    auto stepUs = [&](double resident) {
+      const double busy = resident * t.stepPerGroup;
+      return busy > t.stepAlone ? busy : double(t.stepAlone);
+    };
     for (uint32_t s : kSplitChoices) {
-      if (s > 1 && (kSteps / s < 2 || double(m) * n * s * 4 > double(kWorkspaceBytes))) break;
+      if (s > 1 && (kSteps / s < 1 || double(m) * n * s * 4 > double(kWorkspaceBytes))) break;
       const double groups = tiles * s;
-      double resident = groups / computeUnits;
-      if (resident < 1) resident = 1;
-      if (resident > t.residentGroups) resident = t.residentGroups;
-      // whole rounds: the groups of a partly filled last round take as long as
-      // those of a full one (4097^3 on 256x256 tiles is 289 groups = 2 rounds)
-      const double rounds = std::ceil(groups / (double(computeUnits) * resident) - 1e-9);
-      const double stepUs = resident * mfmaUs > 1.3 ? resident * mfmaUs : 1.3;
-      double us = rounds * ((kSteps + s - 1) / s) * stepUs + 3.0;
+      const double perRound = double(computeUnits) * t.residentGroups;
+      const double fullRounds = std::floor(groups / perRound + 1e-9);
+      const double rest = groups - fullRounds * perRound;
+      double perStep = fullRounds * stepUs(t.residentGroups);
+      if (rest > 0.5) perStep += stepUs(std::ceil(rest / computeUnits - 1e-9));
+      double us = ((kSteps + s - 1) / s) * perStep + 4.0 + 2.5 * t.stepAlone;
       if (s > 1) us += 4.0 + double(m) * n * 4.0 * (s + 1) / 3.0e6;
       if (us < bestUs) {
         bestUs = us;
@@ -463,9 +530,16 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
 } // namespace
 
 namespace {
+constexpr int kConfigCount = int(sizeof(kConfigs) / sizeof(kConfigs[0]));
+static_assert(kConfigCount == POLAR_HIP_MATMUL_TILE_CONFIGS, "the header states how many there are");
+
+// forced: a tile configuration and split count given by the caller instead of
+// the planner's (config < 0: the planner, and the short-contraction kernels
+// where they apply)
 int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const float* a,
                        const float* b, float* c, uint64_t m, uint64_t n, uint64_t k,
-                       int epilogue, const float* bias, float scaleAcc, float scaleBias) {
+                       int epilogue, const float* bias, float scaleAcc, float scaleBias,
+                       MatmulPlan forced = MatmulPlan{-1, 1}) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   if (m == 0 || n == 0) return POLAR_HIP_OK;
   POLAR_HIP_REQUIRE(c != nullptr, "null output");
@@ -489,15 +563,20 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   // short contraction, one long and one short output dimension: streamed in one
   // shot per block (matmul_small_k.hip)
   const MatmulCall call{a, b, c, p.M, p.N, p.K, ta, tb, epilogue, bias, scaleAcc, scaleBias};
-  if (smallKMatmulApplies(call)) return launchSmallKMatmul(dev, call);
-  const MatmulPlan plan = planMatmul(p.M, p.N, p.K, dev->info.compute_units);
+  if (forced.config < 0 && smallKMatmulApplies(call)) return launchSmallKMatmul(dev, call);
+  const MatmulPlan plan =
+      forced.config < 0 ? planMatmul(p.M, p.N, p.K, dev->info.compute_units) : forced;
   switch (plan.config) {
-  case 0: return launchTile<256, 256, 32, 4, 4>(dev, ta, tb, p, plan.splits);
-  case 1: return launchTile<128, 128, 16, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 2: return launchTile<64, 64, 16, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 3: return launchTile<128, 32, 32, 4, 1>(dev, ta, tb, p, plan.splits);
-  case 4: return launchTile<32, 128, 32, 1, 4>(dev, ta, tb, p, plan.splits);
-  default: return launchTile<32, 32, 32, 1, 1>(dev, ta, tb, p, plan.splits);
+  case 0: return launchTile<256, 256, 32, 4, 4, 1>(dev, ta, tb, p, plan.splits);
+  case 1: return launchTile<128, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
+  case 2: return launchTile<64, 64, 32, 2, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 3: return launchTile<128, 32, 32, 4, 1, 2>(dev, ta, tb, p, plan.splits);
+  case 4: return launchTile<32, 128, 32, 1, 4, 2>(dev, ta, tb, p, plan.splits);
+  case 5: return launchTile<32, 32, 32, 1, 1, 1>(dev, ta, tb, p, plan.splits);
+  case 6: return launchTile<256, 128, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits);
+  case 7: return launchTile<128, 256, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
+  case 8: return launchTile<128, 64, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits);
+  default: return launchTile<64, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
   }
 }
 } // namespace
@@ -506,6 +585,44 @@ extern "C" int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
                                  const float* a, const float* b, float* c,
                                  uint64_t m, uint64_t n, uint64_t k) {
   return matmulWithEpilogue(dev, transA, transB, a, b, c, m, n, k, kEpiNone, nullptr, 1.0f, 1.0f);
+}
+
+extern "C" int polar_hip_fmatmul_plan(polar_hip_device* dev, uint64_t m, uint64_t n, uint64_t k,
+                                      int* tile_config, uint32_t* splits, uint32_t tile[3]) {
+  POLAR_HIP_REQUIRE(dev != nullptr && tile_config != nullptr && splits != nullptr, "null argument");
+  POLAR_HIP_REQUIRE(m != 0 && n != 0 && k != 0, "empty product");
+  POLAR_HIP_REQUIRE(m < (1ull << 31) && n < (1ull << 31) && k < (1ull << 31),
+                    "dimension does not fit 31 bits");
+  // the short-contraction kernels take any layout of such a shape
+  const MatmulCall call{nullptr, nullptr, nullptr, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
+                        static_cast<uint32_t>(k), false, false, kEpiNone, nullptr, 1.0f, 1.0f};
+  if (smallKMatmulApplies(call)) {
+    *tile_config = -1;
+    *splits = 1;
+    if (tile != nullptr) tile[0] = tile[1] = tile[2] = 0;
+    return POLAR_HIP_OK;
+  }
+  const MatmulPlan plan = planMatmul(call.M, call.N, call.K, dev->info.compute_units);
+  *tile_config = plan.config;
+  *splits = plan.splits;
+  if (tile != nullptr) {
+    tile[0] = kConfigs[plan.config].bm;
+    tile[1] = kConfigs[plan.config].bn;
+    tile[2] = kConfigs[plan.config].bk;
+  }
+  return POLAR_HIP_OK;
+}
+
+extern "C" int polar_hip_fmatmul_with_plan(polar_hip_device* dev, int transA, int transB,
+                                           const float* a, const float* b, float* c, uint64_t m,
+                                           uint64_t n, uint64_t k, int tile_config,
+                                           uint32_t splits) {
+  POLAR_HIP_REQUIRE(tile_config >= 0 && tile_config < kConfigCount, "no such tile configuration");
+  POLAR_HIP_REQUIRE(splits >= 1 && splits <= 256, "split count out of range");
+  POLAR_HIP_REQUIRE(splits == 1 || m * n * splits * sizeof(float) <= kWorkspaceBytes,
+                    "partial products exceed the workspace");
+  return matmulWithEpilogue(dev, transA, transB, a, b, c, m, n, k, kEpiNone, nullptr, 1.0f, 1.0f,
+                            MatmulPlan{tile_config, splits});
 }
 
 extern "C" int polar_hip_fmatmul_fsigmoid(polar_hip_device* dev, int transA, int transB,

@@ -214,6 +214,48 @@ def test_matmul_unaligned_base(dev, ta, tb):
     assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
 
 
+# every tile configuration of the tiled kernel, whatever the planner would pick: a shape
+# that is a multiple of no tile (edges), one that every tile divides (no edge code), one
+# whose leading dimensions are no multiple of 4 (scalar fetches); one part and split
+TILE_CASES = [(300, 270, 200), (512, 512, 128), (259, 301, 67)]
+
+
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("config", range(10))
+def test_matmul_every_tile_configuration(dev, ta, tb, config):
+    for (m, n, k) in TILE_CASES:
+        _say("tile configuration", config, ta, tb, (m, n, k))
+        rng = np.random.default_rng(config * 131 + m + 2 * ta + tb)
+        sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+        # small integers: exact in fp32 in any order of the additions
+        a = rng.integers(-8, 9, sa).astype(np.float32)
+        b = rng.integers(-8, 9, sb).astype(np.float32)
+        ref = o.fmatmul(ta, tb, a, b)
+        da, db = dev.array(a), dev.array(b)
+        for splits in (1, 3):
+            dc = dev.array(np.full(m * n, np.nan, dtype=np.float32))
+            dev.fmatmul_with_plan(ta, tb, da, db, dc, m, n, k, config, splits)
+            assert np.array_equal(dc.download((m, n)), ref), (config, (m, n, k), splits)
+            dc.free()
+        da.free()
+        db.free()
+
+
+def test_matmul_plan_is_reported_and_forced_plans_are_checked(dev):
+    config, splits, tile = dev.fmatmul_plan(4096, 4096, 4096)
+    assert (config, splits, tile) == (0, 1, (256, 256, 32))
+    config, splits, tile = dev.fmatmul_plan(256, 10, 784)
+    assert 0 <= config < 10 and splits > 1 and tile[2] == 32
+    assert dev.fmatmul_plan(65536, 33, 127)[0] == -1          # the short-contraction kernels
+    x, y, z = dev.empty(64 * 64), dev.empty(64 * 64), dev.empty(64 * 64)
+    for bad in ((10, 1), (-1, 1), (2, 0), (2, 257)):
+        with pytest.raises(Exception):
+            dev.fmatmul_with_plan(False, False, x, y, z, 64, 64, 64, *bad)
+    for t in (x, y, z):
+        t.free()
+
+
 # short contraction with one long and one short output dimension: the one-shot
 # kernels that keep all of K and of the short dimension in LDS (tall: M long,
 # wide: N long), every layout, ragged edges, K and N that are no multiple of 4/16
