@@ -29,6 +29,9 @@
 //    strips of 64 rows, 128-130 us; 256 columns with 1024 lanes and strips of
 //    512 rows (fewer, longer-lived groups), 134 us, and 114 instead of 78 us on
 //    50000 x 1000; strips of 32 rows 151 us (every tile is then read twice);
+//    two tiles in flight per lane instead of one (the tile two steps ahead
+//    fetched into a second register set) 150 us, 132-135 us with strips of
+//    128-256 rows: more outstanding requests make this pattern slower;
 //    numbering the groups strips-first instead of column-tiles-first 131-138
 //    us.  Only 16384^2 prefers the long strips (445 against 482 us).  The
 //    strip's last tile is read by the next strip as well; that second read
