@@ -685,8 +685,9 @@ def test_pool_bit_exact(dev, shape, window, stride):
     x = parity.normal(rng, shape)
     x[0, 0] = -3e6                                     # below the -10e5 floor
     ref = o.fpool(x, window, stride)
-    for mis in (0, 9):
-        dx, dout = dev.array(x), dev.empty(ref.size + 64, mis)
+    # output at and off a line; input rows on 16 bytes (staged by vectors where the width allows) and off them
+    for mis, mis_in in ((0, 0), (9, 0), (0, 3)):
+        dx, dout = dev.array(x, mis_in), dev.empty(ref.size + 64, mis)
         dev.ffill(-7.0, dout)
         dev.fpool(dx, dout, shape[0], shape[1], window, stride)
         got = dout.download()
