@@ -727,14 +727,15 @@ def bench_graphs():
     for key, pinned in (("mlp_forward_backward", False), ("mlp_forward_backward_plugin_ram", True)):
         with harness.Harness(plugin=LIB_PLUGIN, plugin_host_memory=pinned) as h:
             tensors = {}
-            times = {}
+            times, spread = {}, {}
             for graph in (f, gr, u):
                 graphs.emit(graph, h, tensors)
                 h.run()  # first evaluation allocates
                 ts = []
-                for _ in range(3):
+                for _ in range(7):
                     t0 = time.perf_counter(); h.run(); ts.append(time.perf_counter() - t0)
                 times[graph.name] = float(np.median(ts))
+                spread[graph.name] = [round(min(ts) * 1e3, 3), round(max(ts) * 1e3, 3)]
                 h.clear_program()
             out[key] = {
                 "workload": "batch 1024, 1024->4096->1024, sigmoid, logloss; forward, the framework's gradient "
@@ -743,9 +744,10 @@ def bench_graphs():
                 "forward_ms": round(times["mlp_forward"] * 1e3, 3),
                 "gradient_ms": round(times["mlp_gradient"] * 1e3, 3),
                 "update_ms": round(times["mlp_update"] * 1e3, 3),
+                "min_max_ms": spread,  # of the 7 evaluations whose median is reported
                 "nodes": {gph.name: len(gph.nodes) for gph in (f, gr, u)}}
             log(f"{key}: forward {times['mlp_forward'] * 1e3:.2f} ms, gradient "
-                f"{times['mlp_gradient'] * 1e3:.2f} ms, update {times['mlp_update'] * 1e3:.2f} ms")
+                f"{times['mlp_gradient'] * 1e3:.2f} ms, update {times['mlp_update'] * 1e3:.2f} ms  (min, max: {spread})")
     return out
 
 
