@@ -19,7 +19,11 @@
 //     contiguous piece of memory, written within a few hundred cycles, so the
 //     partial lines merge in L2.
 // Waves do not wait for each other, so with 16-24 of them per CU the fetch of
-// one overlaps the arithmetic of the others.  The result does not depend on
+// one overlaps the arithmetic of the others.  Two groups of k in flight per
+// wave is what measured best: with four, 65536 x 33 x 127 goes from 18.0 to
+// 19.6 us and 65536 x 127 x 33 from 18.6 to 23 us; dropping the two fetches
+// that are issued beyond the end of a slice (a peeled last pair) changes
+// nothing for those shapes and costs 33 x 65536 x 127 three microseconds.  The result does not depend on
 // scheduling: every element is accumulated by one lane in k order.
 #include "internal.h"
 #include "matmul_epilogue.h"
