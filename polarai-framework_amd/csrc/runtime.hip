@@ -629,10 +629,19 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
     // destination inside a block of polar_hip_host_alloc: written directly, and
     // complete when the call returns (this handle's own earlier transfers out
     // of the block are ahead of the new one on its stream)
-    std::lock_guard<std::mutex> g(g_hostMu);
-    if (HostBlock* b = hostBlockOf(dst_host, bytes)) {
-      POLAR_HIP_TRY(queueDirect(dev, *b, dst_host, src_device, bytes, hipMemcpyDeviceToHost));
-      POLAR_HIP_TRY(waitForBlock(*b));
+    uint64_t number = 0;
+    {
+      std::lock_guard<std::mutex> g(g_hostMu);
+      if (HostBlock* b = hostBlockOf(dst_host, bytes)) {
+        POLAR_HIP_TRY(queueDirect(dev, *b, dst_host, src_device, bytes, hipMemcpyDeviceToHost));
+        number = b->number;
+      }
+    }
+    if (number != 0) {
+      // wait outside the table's lock (a large read-back takes milliseconds);
+      // the block learns that it is idle from the device's count
+      POLAR_HIP_TRY(hipStreamSynchronize(dev->stream));
+      dev->noteDirectDone(number);
       return POLAR_HIP_OK;
     }
   }
