@@ -344,16 +344,25 @@ __global__ __launch_bounds__(kSegment) void poolStagedKernel(PoolStagedArgs q) {
     const int64_t xa = x0 - int64_t(q.lead); // multiple of 4, like W: a vector is inside the image or outside
     const float* const rowBase = p.in + uint64_t(y0) * p.stride0 * p.W;
     constexpr int kVecBatch = 8;
+    // row and column of the lane's vector move on by 256 vectors per load: one
+    // division per lane instead of one per load
+    const uint32_t stepRow = uint32_t(kSegment) / perRow, stepCol = uint32_t(kSegment) % perRow;
+    uint32_t row = t / perRow, c = t - row * perRow;
     for (uint32_t first = 0; first < vectors; first += kSegment * kVecBatch) {
       v4f v[kVecBatch];
 #pragma unroll
       for (int u = 0; u < kVecBatch; ++u) {
         const uint32_t idx = first + t + u * kSegment;
-        const uint32_t row = idx / perRow, c = idx - row * perRow;
         const int64_t xi = xa + 4 * int64_t(c);
         v[u] = (idx < vectors && xi >= 0 && xi < int64_t(p.W))
                    ? *reinterpret_cast<const v4f*>(rowBase + uint64_t(row) * p.W + xi)
                    : v4f{0.f, 0.f, 0.f, 0.f};
+        row += stepRow;
+        c += stepCol;
+        if (c >= perRow) {
+          c -= perRow;
+          ++row;
+        }
       }
 #pragma unroll
       for (int u = 0; u < kVecBatch; ++u) {
