@@ -166,6 +166,14 @@ __device__ __forceinline__ void streamStore(polar_v4f value, polar_v4f* address)
 __device__ __forceinline__ void streamStore(float value, float* address) {
   asm volatile("global_store_dword %0, %1, off sc1 nt" : : "v"(address), "v"(value) : "memory");
 }
+// the same, kByteOffset (0 .. 4095) bytes behind `address`: the offset travels
+// in the instruction, so several stores share one address computation
+template <int kByteOffset>
+__device__ __forceinline__ void streamStoreAt(float value, float* address) {
+  static_assert(kByteOffset >= 0 && kByteOffset < 4096, "offset field of the store");
+  asm volatile("global_store_dword %0, %1, off offset:%2 sc1 nt"
+               : : "v"(address), "v"(value), "n"(kByteOffset) : "memory");
+}
 
 inline bool aligned16(const void* p) {
   return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;

@@ -60,6 +60,7 @@ constexpr int kLine = 32;     // floats per 128-byte line
 constexpr int kConvRows = 12; // output rows per fconv2d work-group
 constexpr int kPoolRows = 2;  // output rows per fpool work-group
 constexpr uint32_t kMaxConvLds = 64 * 1024;
+constexpr int kWaitVmcnt0 = 0x0F70; // s_waitcnt vmcnt(0) with the other counters left alone
 constexpr uint32_t kMaxPoolLds = 24 * 1024; // window of the staged fpool kernel: six groups per CU
 constexpr uint32_t kPoolStagedRows = 12;    // output rows per group of that kernel, at most
 
@@ -89,8 +90,21 @@ struct ConvArgs {
   uint32_t outPhase; // (address of out / 4) mod 32
 };
 
-// KH_/KW_ == 0: the kernel size comes from the arguments.
-template <int KH_, int KW_>
+// Columns of the staged window: the 256 + 31 + KW - 1 the band needs and, when
+// the image rows start on 16 bytes (VEC), one more in front and padding to a
+// whole number of 16-byte vectors.  The first column a band needs is
+// 256 ct - 31; one column earlier is a multiple of 32: the window then starts
+// on a line of its image row.
+constexpr uint32_t kConvLead = 1;
+__host__ __device__ constexpr uint32_t convPitch(uint32_t kw, bool vec) {
+  return vec ? (kConvLead + kSegment + (kLine - 1) + kw - 1 + 3) / 4 * 4
+             : kSegment + (kLine - 1) + kw - 1;
+}
+
+// KH_/KW_ == 0: the kernel size comes from the arguments.  VEC: image rows
+// start on 16 bytes (the host checks); full bands inside the image are then
+// staged with 16-byte loads.
+template <int KH_, int KW_, bool VEC>
 __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   extern __shared__ float tile[];
   const uint32_t KH = KH_ ? KH_ : p.KH, KW = KW_ ? KW_ : p.KW;
@@ -100,16 +114,53 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   const uint32_t y0 = rt * kConvRows;
   const uint32_t rowsOut = p.OH - y0 < uint32_t(kConvRows) ? p.OH - y0 : uint32_t(kConvRows);
   const uint32_t rowsIn = rowsOut + KH - 1; // all inside the input: OH = H - KH + 1
-  const uint32_t pitch = kSegment + (kLine - 1) + KW - 1;
-  // input column held in tile column 0 (may be negative in the first segment)
-  const int64_t x0 = int64_t(ct) * kSegment - (kLine - 1);
+  const uint32_t pitch = convPitch(KW, VEC);
+  constexpr uint32_t lead = VEC ? kConvLead : 0;
+  // input column held in tile column 0 (may be negative in the first segment);
+  // the first column the band needs is `lead` columns further on
+  const int64_t x0 = int64_t(ct) * kSegment - (kLine - 1) - lead;
 
   // Stage the window: lane t takes elements t, t+256, ... of the window in
   // row-major order.  pitch > 256, so stepping by 256 wraps to the next row at
   // most once.
   const uint32_t t = threadIdx.x;
   bool staged = false;
-  if constexpr (KH_ != 0) {
+  if constexpr (KH_ != 0 && VEC) {
+    // Full band of a constant-size kernel, window inside the image, rows on 16
+    // bytes: lane t takes vectors t, t+256, ... of the window in row-major order.
+    // Row and column of a vector are those of the lane's first one plus
+    // constants and one compare; all loads are issued before the first LDS
+    // store.  A quarter of the load instructions of the dword path below, and
+    // a third of its address arithmetic.
+    constexpr uint32_t P4 = convPitch(KW_ ? KW_ : 1, true) / 4; // vectors per window row
+    constexpr uint32_t kRows = kConvRows + KH_ - 1;
+    constexpr uint32_t kVectors = kRows * P4;
+    constexpr int kRounds = (kVectors + kSegment - 1) / kSegment;
+    if (x0 >= 0 && x0 + int64_t(4 * P4) <= int64_t(p.W) && rowsOut == uint32_t(kConvRows) &&
+        uint64_t(kRows) * p.W < (1u << 30)) {
+      const float* base = p.in + uint64_t(y0) * p.W + x0;
+      const uint32_t row0 = t / P4, c0 = t % P4;
+      v4f v[kRounds];
+#pragma unroll
+      for (int u = 0; u < kRounds; ++u) {
+        constexpr uint32_t kStep = kSegment; // vectors between a lane's loads
+        const uint32_t dq = uint32_t(u) * kStep / P4, dr = uint32_t(u) * kStep % P4; // constants after unrolling
+        const bool wrap = c0 + dr >= P4;
+        const uint32_t row = row0 + dq + (wrap ? 1u : 0u);
+        const uint32_t c = c0 + dr - (wrap ? P4 : 0u);
+        if (uint32_t(u + 1) * kStep <= kVectors || uint32_t(u) * kStep + t < kVectors)
+          v[u] = *reinterpret_cast<const v4f*>(base + (row * p.W + 4 * c));
+      }
+#pragma unroll
+      for (int u = 0; u < kRounds; ++u) {
+        constexpr uint32_t kStep = kSegment;
+        if (uint32_t(u + 1) * kStep <= kVectors || uint32_t(u) * kStep + t < kVectors)
+          *reinterpret_cast<v4f*>(tile + 4 * (uint32_t(u) * kStep + t)) = v[u];
+      }
+      staged = true;
+    }
+  }
+  if constexpr (KH_ != 0 && !VEC) {
     // Full band of a constant-size kernel with the whole window inside the
     // image: row and column of every element are compile-time constants plus
     // one compare, nothing is predicated, and all loads are issued before the
@@ -171,6 +222,12 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   } else {
     for (uint32_t i = t; i < KH * KW; i += kSegment) wlds[i] = p.weights[i];
   }
+  // Every load of the staging phase has to be back before the barrier anyway.
+  // Saying so here keeps the compiler from putting its own vmcnt(0) into the row
+  // loop below (it would protect registers of loads whose lanes were
+  // predicated off), where the counter also holds the previous row's stores:
+  // each row would then wait for the stores of the row before.
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
   __syncthreads();
 
   // A wave takes every fourth row of the band; a lane computes the four
@@ -187,11 +244,14 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t / 64), lane = t % 64;
   const int32_t xLane = int32_t(ct * kSegment + lane); // before the row's shift
   const int32_t ow = int32_t(p.OW);
+  // segments whose 256 columns exist for every shift a row can have (0 .. 31):
+  // no lane of the group needs a bounds check
+  const bool interior = ct >= 1 && uint64_t(ct) * kSegment + kSegment <= p.OW;
   for (uint32_t r = wave; r < rowsOut; r += kSegment / 64) {
     const uint32_t y = y0 + r;
     const uint32_t shift = rowShift(y, p.OW, p.outPhase);
     const int32_t x = xLane - int32_t(shift); // the lane's first output; the others 64 apart
-    const float* win = tile + r * pitch + (kLine - 1) - shift + lane;
+    const float* win = tile + r * pitch + lead + (kLine - 1) - shift + lane;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     for (uint32_t a = 0; a < KH; ++a)
       for (uint32_t b = 0; b < KW; ++b) {
@@ -202,10 +262,19 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
         for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + 64 * j] * wt + acc[j];
       }
     float* const rowOut = p.out + uint64_t(y) * p.OW; // scalar
+    if (interior) {
+      // every lane's four outputs exist: one address, the others by offset
+      float* const o = rowOut + x;
+      streamStoreAt<0>(acc[0], o);
+      streamStoreAt<256>(acc[1], o);
+      streamStoreAt<512>(acc[2], o);
+      streamStoreAt<768>(acc[3], o);
+    } else {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int32_t xj = x + 64 * j;
-      if (xj >= 0 && xj < ow) streamStore(acc[j], rowOut + xj);
+      for (int j = 0; j < 4; ++j) {
+        const int32_t xj = x + 64 * j;
+        if (xj >= 0 && xj < ow) streamStore(acc[j], rowOut + xj);
+      }
     }
   }
 }
@@ -288,6 +357,12 @@ __global__ __launch_bounds__(kSegment) void poolSquareKernel(PoolArgs p) {
     for (int a = 0; a < WIN; ++a)
       v[r][a] = *reinterpret_cast<const vw*>(corner + uint64_t(a) * p.W);
   }
+  // All of the band's loads are waited for here, in one go.  Left to itself the
+  // compiler waits for each row's loads just before that row's compares, by
+  // count; the streaming stores below are in that count too (and unknown to
+  // the compiler, being asm), so the second row's wait would also wait for the
+  // first row's store to come back.
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
 #pragma unroll
   for (int r = 0; r < kPoolRows; ++r) {
     float best = -10e5f;
@@ -398,6 +473,7 @@ __global__ __launch_bounds__(kSegment) void poolStagedKernel(PoolStagedArgs q) {
     for (int u = 0; u < kBatch; ++u)
       if (idx + u * kSegment < total) tile[idx + u * kSegment] = v[u];
   }
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0); // as in conv2dKernel: no vmcnt(0) of the compiler's in the row loop
   __syncthreads();
 
   const uint32_t wave = __builtin_amdgcn_readfirstlane(t / 64), lane = t % 64;
@@ -477,17 +553,17 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in, const float* kerne
   p.colTiles = (p.OW + (kLine - 1) + kSegment - 1) / kSegment;
   p.outPhase = phaseOf(out);
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
-  const uint64_t ldsBytes = (uint64_t(kConvRows + p.KH - 1) *
-                                 (kSegment + (kLine - 1) + p.KW - 1) +
+  const bool vec = p.W % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0;
+  const uint64_t ldsBytes = (uint64_t(kConvRows + p.KH - 1) * convPitch(p.KW, vec) +
                              uint64_t(p.KH) * p.KW) * sizeof(float); // window + weights
   if (ldsBytes <= kMaxConvLds) {
     const uint64_t tiles = uint64_t(p.colTiles) * ((p.OH + kConvRows - 1) / kConvRows);
     POLAR_HIP_REQUIRE(tiles < (1ull << 31) - kXcds, "tensor too large for one launch");
     p.tiles = static_cast<uint32_t>(tiles);
     const uint64_t grid = paddedGrid(tiles);
-    auto fn = p.KH == 3 && p.KW == 3   ? conv2dKernel<3, 3>
-              : p.KH == 5 && p.KW == 5 ? conv2dKernel<5, 5>
-                                       : conv2dKernel<0, 0>;
+    auto fn = p.KH == 3 && p.KW == 3   ? (vec ? conv2dKernel<3, 3, true> : conv2dKernel<3, 3, false>)
+              : p.KH == 5 && p.KW == 5 ? (vec ? conv2dKernel<5, 5, true> : conv2dKernel<5, 5, false>)
+                                       : (vec ? conv2dKernel<0, 0, true> : conv2dKernel<0, 0, false>);
     POLAR_HIP_TRY(launchKernelLds(dev, fn, dim3(static_cast<unsigned>(grid)),
                                   dim3(kSegment), static_cast<uint32_t>(ldsBytes), p));
   } else {
