@@ -49,6 +49,9 @@
 //    fall back to taps from memory.
 #include "internal.h"
 
+#include <type_traits>
+#include <utility>
+
 using namespace polar_hip_detail;
 
 namespace {
@@ -99,6 +102,31 @@ constexpr uint32_t kConvLead = 1;
 __host__ __device__ constexpr uint32_t convPitch(uint32_t kw, bool vec) {
   return vec ? (kConvLead + kSegment + (kLine - 1) + kw - 1 + 3) / 4 * 4
              : kSegment + (kLine - 1) + kw - 1;
+}
+
+// LDS reads with the distance from a base address in the instruction (up to 64
+// KB), for unrolled taps.  The compiler does not know what the asm does, so
+// the wait for the data is explicit: ldsReadsDone takes the values as operands,
+// which keeps every use of them behind it.
+__device__ __forceinline__ uint32_t ldsAddress(const float* p) {
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (const __attribute__((address_space(3))) float*)(p)));
+}
+template <uint32_t kByteOffset>
+__device__ __forceinline__ float ldsReadAt(uint32_t address) {
+  static_assert(kByteOffset < 65536, "offset field of the LDS read");
+  float v;
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(address), "n"(kByteOffset));
+  return v;
+}
+template <int... I, typename F>
+__device__ __forceinline__ void forEachConstant(std::integer_sequence<int, I...>, F f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+__device__ __forceinline__ void ldsReadsDone(float (&v)[4][3]) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(v[0][0]), "+v"(v[0][1]), "+v"(v[0][2]), "+v"(v[1][0]), "+v"(v[1][1]), "+v"(v[1][2]),
+                 "+v"(v[2][0]), "+v"(v[2][1]), "+v"(v[2][2]), "+v"(v[3][0]), "+v"(v[3][1]), "+v"(v[3][2]));
 }
 
 // KH_/KW_ == 0: the kernel size comes from the arguments.  VEC: image rows
@@ -253,14 +281,40 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
     const int32_t x = xLane - int32_t(shift); // the lane's first output; the others 64 apart
     const float* win = tile + r * pitch + lead + (kLine - 1) - shift + lane;
     float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (uint32_t a = 0; a < KH; ++a)
-      for (uint32_t b = 0; b < KW; ++b) {
-        float wt;
-        if constexpr (KH_ != 0) wt = wreg[a * KW_ + b];
-        else wt = wlds[a * KW + b];
+    if constexpr (KH_ == 3 && KW_ == 3) {
+      // The 36 taps of the lane's four outputs, each read with its distance from
+      // `win` in the instruction's offset field.  Written in C the compiler
+      // pairs the reads (ds_read2, whose offsets reach 1 KB only) and spends a
+      // vector add per pair on addresses: 6 of the 24 vector instructions per
+      // output, in a kernel whose duration follows its instruction count.
+      constexpr uint32_t P = convPitch(3, VEC);
+      const uint32_t at = ldsAddress(win);
+      float v[3][4][3];
+      forEachConstant(std::make_integer_sequence<int, 12>{}, [&](auto index) {
+        constexpr int a = decltype(index)::value / 4, j = decltype(index)::value % 4;
+        v[a][j][0] = ldsReadAt<(a * P + 64 * j + 0) * 4>(at);
+        v[a][j][1] = ldsReadAt<(a * P + 64 * j + 1) * 4>(at);
+        v[a][j][2] = ldsReadAt<(a * P + 64 * j + 2) * 4>(at);
+      });
+      ldsReadsDone(v[0]);
+      ldsReadsDone(v[1]);
+      ldsReadsDone(v[2]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + 64 * j] * wt + acc[j];
-      }
+      for (int a = 0; a < 3; ++a)
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] = v[a][j][b] * wreg[a * 3 + b] + acc[j];
+    } else {
+      for (uint32_t a = 0; a < KH; ++a)
+        for (uint32_t b = 0; b < KW; ++b) {
+          float wt;
+          if constexpr (KH_ != 0) wt = wreg[a * KW_ + b];
+          else wt = wlds[a * KW + b];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] = win[a * pitch + b + 64 * j] * wt + acc[j];
+        }
+    }
     float* const rowOut = p.out + uint64_t(y) * p.OW; // scalar
     if (interior) {
       // every lane's four outputs exist: one address, the others by offset
