@@ -17,7 +17,9 @@
 //    product rounded before the add (the file is compiled with
 //    -ffp-contract=off).  3x3 and 5x5 are compiled with constant bounds.
 //    Measured on an 8192^2 image, 3x3, buffers rotated (537 MB per launch; a
-//    plain copy of that size takes 80 us): 93 us.  HBM traffic is 1.002 x the
+//    plain copy of that size takes 80 us): 89 us (93 us before the staging by
+//    vectors, the unchecked interior stores, the offset LDS reads and the
+//    explicit wait described at those places).  HBM traffic is 1.002 x the
 //    algorithmic bytes and the LDS reads are free of bank conflicts; the
 //    counters show the waves parked at the barrier, waiting for the window,
 //    for most of their life (with the arithmetic removed the kernel still
