@@ -29,7 +29,9 @@
 //    that the reads stay conflict-free, 16-byte staging loads), no LDS at all
 //    (a lane fetching its own KW+3 inputs per tap row: 98-110 us), a resident
 //    grid of groups that prefetch their next band into registers while they
-//    compute (116 us in row-major band order, 152 us walking down strips), a
+//    compute (116 us in row-major band order, 152 us walking down strips; two
+//    bands per group, one below the other, the second window on its way into
+//    registers while the first is computed: 97 us against 89), a
 //    window per wave instead of per group, without any group barrier and with
 //    the first output rows computed while the later window rows are still in
 //    flight (105-142 us for 2-8 rows per wave), 16 or more rows per band
