@@ -143,7 +143,10 @@ def test_in_place_update(dev):
 
 @pytest.mark.parametrize("shape", [(1, 1), (1, 7), (7, 1), (3, 5), (64, 64), (65, 63), (64, 1000),
                                    (1000, 64), (257, 129), (1031, 517), (1, 100003), (100003, 1),
-                                   (513, 1025), (2048, 2048), (127, 4099), (4099, 127), (12345, 6789)])
+                                   (513, 1025), (2048, 2048), (127, 4099), (4099, 127), (12345, 6789),
+                                   # output pitch a large power-of-two multiple (strips numbered in runs),
+                                   # with full and ragged column tiles; interior strips on the lean path
+                                   (8192, 300), (10240, 257), (16384, 128), (2048, 4100), (300, 8192)])
 def test_transpose(dev, shape):
     _say("transpose", shape)
     rng = np.random.default_rng(shape[0] * 7919 + shape[1])
