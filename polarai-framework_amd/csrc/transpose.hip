@@ -26,7 +26,7 @@
 //    TB/s); the stores, which never share a line, stay non-temporal.
 //  * Shape, measured with rotated buffers on 12345 x 6789 (and seven other
 //    shapes from 333 x 777 to 16384^2): column tiles of 128 with 512 lanes and
-//    strips of 64 rows, 128-130 us; 256 columns with 1024 lanes and strips of
+//    strips of 64 rows, 128-130 us (125.5-126.5 us with the interior path); 256 columns with 1024 lanes and strips of
 //    512 rows (fewer, longer-lived groups), 134 us, and 114 instead of 78 us on
 //    50000 x 1000; strips of 32 rows 151 us (every tile is then read twice);
 //    two tiles in flight per lane instead of one (the tile two steps ahead
