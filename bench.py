@@ -514,6 +514,33 @@ def bench_copies(dev):
         log(f"copy {label:8s}: to device {up * 1e6:9.1f} us ({nbytes / up / 1e9:6.2f} GB/s), "
             f"to host {down * 1e6:9.1f} us ({nbytes / down / 1e9:6.2f} GB/s)")
         buf.free()
+        # the same transfers out of and into a pinned block of the library (no staging)
+        block = dev.host_alloc(nbytes)
+        try:
+            import ctypes
+            pinned = np.ctypeslib.as_array(ctypes.cast(block, ctypes.POINTER(ctypes.c_float)), shape=(nbytes // 4,))
+            pinned[:] = 1.0
+            buf = dev.empty(nbytes // 4)
+            for _ in range(2):
+                dev.copy_to_device(buf.ptr, block, nbytes); dev.copy_to_host(block, buf.ptr, nbytes)
+            dev.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                dev.copy_to_device(buf.ptr, block, nbytes)   # returns with the transfer queued
+            dev.synchronize()
+            up = (time.perf_counter() - t0) / reps
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                dev.copy_to_host(block, buf.ptr, nbytes)
+            down = (time.perf_counter() - t0) / reps
+            assert pinned[0] == 1.0 and pinned[-1] == 1.0
+            out[label + " pinned block"] = {"to_device_us": round(up * 1e6, 1), "to_device_GB/s": round(nbytes / up / 1e9, 2),
+                                            "to_host_us": round(down * 1e6, 1), "to_host_GB/s": round(nbytes / down / 1e9, 2)}
+            log(f"     pinned : to device {up * 1e6:9.1f} us ({nbytes / up / 1e9:6.2f} GB/s), "
+                f"to host {down * 1e6:9.1f} us ({nbytes / down / 1e9:6.2f} GB/s)")
+            buf.free()
+        finally:
+            dev.host_free(block)
     return out
 
 
