@@ -636,7 +636,10 @@ def test_softmax_is_repeatable(dev):
 
 CONV_SHAPES = [((4, 4), (3, 3)), ((3, 3), (3, 3)), ((37, 53), (3, 3)), ((300, 1000), (5, 5)),
                ((129, 700), (7, 3)), ((64, 64), (1, 1)), ((1, 515), (1, 3)), ((515, 1), (3, 1)),
-               ((40, 300), (23, 23)), ((100, 2049), (3, 5)), ((33, 289), (9, 1))]
+               ((40, 300), (23, 23)), ((100, 2049), (3, 5)), ((33, 289), (9, 1)),
+               # rows on 16 bytes and several column segments: bands staged by vectors, interior segments
+               # stored without bounds checks, ragged last band
+               ((40, 1024), (3, 3)), ((25, 2052), (3, 3)), ((13, 600), (3, 3)), ((50, 1536), (5, 5))]
 
 
 @pytest.mark.parametrize("shape,kshape", CONV_SHAPES)
