@@ -18,7 +18,7 @@
 //   * A wave stores its accumulators directly; its 16 rows of C are one
 //     contiguous piece of memory, written within a few hundred cycles, so the
 //     partial lines merge in L2.
-// Waves do not wait for each other, so with 16-24 of them per CU the fetch of
+// Waves do not wait for each other, so with 16 of them per CU the fetch of
 // one overlaps the arithmetic of the others.  Two groups of k in flight per
 // wave is what measured best: with four, 65536 x 33 x 127 goes from 18.0 to
 // 19.6 us and 65536 x 127 x 33 from 18.6 to 23 us; dropping the two fetches
@@ -35,9 +35,8 @@ namespace {
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t kMaxK = 128;
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * 64;
-constexpr int kBlock = kWaves * 16; // values of the long dimension per work-group and turn
+// A work-group has WAVES waves (4 or 8, a template parameter below): 64 WAVES
+// lanes, and 16 WAVES values of the long dimension per turn.
 
 struct SmallKArgs {
   const float* A;
@@ -73,6 +72,7 @@ struct ShortTile {
     return (KCONTIG ? xPadded : k4) * pitchFor(xPadded, k4);
   }
 
+  template <int kThreads>
   static __device__ __forceinline__ void load(float* S, const float* X, uint32_t xdim,
                                               uint32_t xPadded, uint32_t K, uint32_t k4,
                                               uint32_t pitch, int t) {
@@ -123,8 +123,10 @@ __device__ __forceinline__ void storeResult(const SmallKArgs& p, size_t idx, flo
 // TS blocks of 16 cover the short dimension.  TALL: M is the long dimension (B
 // is the short operand, N <= 16*TS); otherwise N is (A is the short operand,
 // M <= 16*TS).
-template <int TS, bool TA, bool TB, bool TALL>
-__global__ __launch_bounds__(kThreads) void smallKKernel(SmallKArgs p) {
+template <int TS, bool TA, bool TB, bool TALL, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void smallKKernel(SmallKArgs p) {
+  constexpr int kThreads = WAVES * 64;
+  constexpr int kBlock = WAVES * 16; // values of the long dimension per work-group and turn
   extern __shared__ __attribute__((aligned(16))) float shortS[];
   // A is k-contiguous when not transposed ([M x K]); B when transposed ([N x K])
   constexpr bool kShortKContig = TALL ? TB : !TA;
@@ -179,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void smallKKernel(SmallKArgs p) {
   // brought in: they travel while that happens
   const uint32_t firstX = blockIdx.x * kBlock + wave * 16 + fx;
   v4f next0 = fetchGroup(firstX, 0), next1 = fetchGroup(firstX, 1 < groups ? 1 : lastGroup);
-  Short::load(shortS, TALL ? p.B : p.A, shortDim, TS * 16, p.K, p.k4, p.pitch, t);
+  Short::template load<kThreads>(shortS, TALL ? p.B : p.A, shortDim, TS * 16, p.K, p.k4, p.pitch, t);
   __syncthreads();
 
   for (uint32_t block = blockIdx.x; block < blocks; block += gridDim.x) {
@@ -229,13 +231,14 @@ __global__ __launch_bounds__(kThreads) void smallKKernel(SmallKArgs p) {
   }
 }
 
-template <int TS, bool TA, bool TB, bool TALL>
-int launchConfig(polar_hip_device* dev, SmallKArgs p) {
+template <int TS, bool TA, bool TB, bool TALL, int WAVES>
+int launchWaves(polar_hip_device* dev, SmallKArgs p, uint32_t groupsPerCu) {
   constexpr bool kShortKContig = TALL ? TB : !TA;
   using Short = ShortTile<kShortKContig>;
+  constexpr int kBlock = WAVES * 16;
   p.pitch = Short::pitchFor(TS * 16, p.k4);
   const uint32_t bytes = Short::words(TS * 16, p.k4) * sizeof(float);
-  auto kernel = smallKKernel<TS, TA, TB, TALL>;
+  auto kernel = smallKKernel<TS, TA, TB, TALL, WAVES>;
   // more dynamic LDS than the default limit has to be asked for, once per
   // kernel and device
   static uint64_t raised = 0;
@@ -245,15 +248,27 @@ int launchConfig(polar_hip_device* dev, SmallKArgs p) {
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
     raised |= bit;
   }
-  // one turn per group up to four groups per CU; beyond that groups take
+  // one turn per group up to groupsPerCu groups per CU; beyond that groups take
   // several turns (and load the short operand once for all of them)
   const uint32_t longDim = TALL ? p.M : p.N;
   const uint32_t blocks = (longDim + kBlock - 1) / kBlock;
-  const uint32_t slots = 4u * static_cast<uint32_t>(dev->info.compute_units);
+  const uint32_t slots = groupsPerCu * static_cast<uint32_t>(dev->info.compute_units);
   const uint32_t turns = (blocks + slots - 1) / slots;
   const uint32_t groups = (blocks + turns - 1) / turns;
-  POLAR_HIP_TRY(launchKernelLds(dev, kernel, dim3(groups), dim3(kThreads), bytes, p));
+  POLAR_HIP_TRY(launchKernelLds(dev, kernel, dim3(groups), dim3(WAVES * 64), bytes, p));
   return POLAR_HIP_OK;
+}
+
+// Sixteen waves per CU either way.  Long operands (from 32768 rows or columns)
+// take them as two groups of eight, each loading the short operand once for
+// two turns: 65536 x 33 x 127 18.0 -> 16.7-17.1 us, 33 x 65536 x 127 16.5 ->
+// 15.3-15.8 us.  Shorter ones keep four groups of four (8192 x 128 x 128: 15.8
+// against 17.9 us with eight-wave groups).
+template <int TS, bool TA, bool TB, bool TALL>
+int launchConfig(polar_hip_device* dev, const SmallKArgs& p) {
+  const uint32_t longDim = TALL ? p.M : p.N;
+  if (longDim >= 32768) return launchWaves<TS, TA, TB, TALL, 8>(dev, p, 2);
+  return launchWaves<TS, TA, TB, TALL, 4>(dev, p, 4);
 }
 
 template <int TS, bool TALL>
