@@ -63,7 +63,10 @@ struct TransposeArgs {
   float* out;
   uint32_t rows, cols;
   uint32_t colTiles;        // ceil(cols / kTJ)
-  uint32_t colTilesPerXcd;  // ceil(colTiles / 8)
+  uint32_t colTilesPerXcd;  // colTiles / 8: the column tiles every XCD owns outright
+  uint32_t sharedTiles;     // colTiles % 8: the rest, whose strips are dealt out to the XCDs
+  uint32_t ownedGroups;     // groups per XCD for the tiles it owns (strips rounded up to whole runs)
+  uint32_t stripsPerXcd;    // ceil(strips / 8): an XCD's share of the strips of the shared tiles
   uint32_t strips;          // ceil(rows / stripRows)
   uint32_t stripRows;       // multiple of kTI
   uint32_t fastOffsets;     // rows * cols < 2^31: element offsets fit 32 bits
@@ -74,14 +77,25 @@ __global__ __launch_bounds__(kThreads) void transposeKernel(TransposeArgs p) {
   __shared__ float ring[2 * kTI][kTJ + 1];
 
   // XCD x (work-groups with id % 8 == x) owns column tiles
-  // [x*perXcd, (x+1)*perXcd) and walks them fastest.
+  // [x*perXcd, (x+1)*perXcd) and walks them fastest, in runs of p.run strips
+  // per column tile (1: column tiles fastest).  The colTiles % 8 tiles that are
+  // left over are shared: every XCD takes an eighth of their strips, so that
+  // all XCDs finish together (with 54 column tiles dealt out whole, seven XCDs
+  // would hold 7 and the eighth 5, idle for the last 2/7 of the launch).
   const uint32_t xcd = blockIdx.x % kXcds, local = blockIdx.x / kXcds;
-  // ... in runs of p.run strips per column tile (1: column tiles fastest)
-  const uint32_t perRun = p.run * p.colTilesPerXcd;
-  const uint32_t inRun = local % perRun;
-  const uint32_t colTile = xcd * p.colTilesPerXcd + inRun / p.run;
-  const uint32_t strip = local / perRun * p.run + inRun % p.run;
-  if (colTile >= p.colTiles || strip >= p.strips) return; // before any barrier
+  uint32_t colTile, strip;
+  if (local < p.ownedGroups) {
+    const uint32_t perRun = p.run * p.colTilesPerXcd;
+    const uint32_t inRun = local % perRun;
+    colTile = xcd * p.colTilesPerXcd + inRun / p.run;
+    strip = local / perRun * p.run + inRun % p.run;
+    if (strip >= p.strips) return; // the padding of the last run; before any barrier
+  } else {
+    const uint32_t rest = local - p.ownedGroups; // < sharedTiles * stripsPerXcd
+    colTile = kXcds * p.colTilesPerXcd + rest % p.sharedTiles;
+    strip = xcd * p.stripsPerXcd + rest / p.sharedTiles;
+    if (strip >= p.strips) return;
+  }
 
   const uint32_t R = p.rows, C = p.cols;
   const uint32_t j0 = colTile * kTJ;
@@ -216,7 +230,8 @@ extern "C" int polar_hip_ftranspose(polar_hip_device* dev, const float* in,
   p.rows = static_cast<uint32_t>(rows);
   p.cols = static_cast<uint32_t>(cols);
   p.colTiles = (p.cols + kTJ - 1) / kTJ;
-  p.colTilesPerXcd = (p.colTiles + kXcds - 1) / kXcds;
+  p.colTilesPerXcd = p.colTiles / kXcds;
+  p.sharedTiles = p.colTiles % kXcds;
   // Strips of 64 rows, shorter when that is needed to give every CU two groups.
   const uint64_t wanted = 2ull * static_cast<uint64_t>(dev->info.compute_units);
   uint32_t stripRows = 64;
@@ -233,7 +248,11 @@ extern "C" int polar_hip_ftranspose(polar_hip_device* dev, const float* in,
   // measured 16384^2 495 -> 410 us, 8192 x 6789 92 -> 83 us, 12288^2 253 -> 229
   // us; with an odd pitch (12345 x 6789) runs cost 1-3 %.
   p.run = (p.rows % 2048 == 0 && p.rows >= 8192) ? 16 : 1;
-  const uint64_t grid = uint64_t(kXcds) * p.colTilesPerXcd * ((p.strips + p.run - 1) / p.run * p.run);
+  const uint64_t owned = uint64_t(p.colTilesPerXcd) * ((p.strips + p.run - 1) / p.run * p.run);
+  p.stripsPerXcd = (p.strips + kXcds - 1) / kXcds;
+  const uint64_t grid = uint64_t(kXcds) * (owned + uint64_t(p.sharedTiles) * p.stripsPerXcd);
+  POLAR_HIP_REQUIRE(owned < (1ull << 31), "matrix too large for one launch");
+  p.ownedGroups = static_cast<uint32_t>(owned);
   POLAR_HIP_REQUIRE(grid < (1ull << 31), "matrix too large for one launch");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   POLAR_HIP_TRY(launchKernel(dev, transposeKernel,
