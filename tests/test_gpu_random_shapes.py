@@ -123,3 +123,56 @@ def test_random_matmul_medium(dev, seed):
     assert parity.frobenius_rel_error(got, ref) <= 1e-5
     for t in (da, db, dc):
         t.free()
+
+
+@pytest.mark.parametrize("seed", range(12 * SCALE))
+def test_random_transpose_large(dev, seed):
+    """Shapes with many interior strips and column tiles (the path without bounds checks), column
+    tile counts that do not divide by eight (tiles shared between the XCDs), now and then a row
+    count that numbers the strips in runs."""
+    rng = np.random.default_rng(6500 + seed)
+    rows = int(rng.integers(700, 6000)) if seed % 4 else int(rng.choice([8192, 10240]))
+    cols = int(rng.integers(130, 2500))
+    _say("random large transpose", seed, (rows, cols))
+    x = (np.arange(rows * cols, dtype=np.int64) % 16000057).astype(np.float32).reshape(rows, cols)
+    dx, dt = dev.array(x), dev.empty(x.size + 32)
+    dev.ffill(-7.0, dt)
+    dev.ftranspose(dx, dt, rows, cols)
+    got = dt.download()
+    assert np.array_equal(got[:x.size].reshape(cols, rows), x.T)
+    assert np.all(got[x.size:] == -7.0)
+    dx.free(); dt.free()
+
+
+@pytest.mark.parametrize("seed", range(12 * SCALE))
+def test_random_conv2d_and_pool_wide_rows_on_16_bytes(dev, seed):
+    """Widths that are multiples of 4 and span several column segments: windows staged by vectors,
+    interior segments stored without bounds checks, ragged last bands."""
+    rng = np.random.default_rng(7500 + seed)
+    kh = kw = int(rng.choice([3, 3, 5, 7]))
+    h = int(rng.integers(kh, 90))
+    w = 4 * int(rng.integers(130, 800))
+    mis = int(rng.choice([0, 5]))
+    _say("random wide conv2d", seed, (h, w), (kh, kw), "misalign", mis)
+    x, k = parity.normal(rng, (h, w)), parity.normal(rng, (kh, kw))
+    ref = o.fconv2d(x, k)
+    dx, dk, dout = dev.array(x), dev.array(k), dev.empty(ref.size + 32, mis)
+    dev.ffill(-7.0, dout)
+    dev.fconv2d(dx, dk, dout, h, w, kh, kw)
+    got = dout.download()
+    assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+    assert np.all(got[ref.size:] == -7.0)
+    dout.free(); dk.free()
+
+    win = (int(rng.integers(2, min(h, 5) + 1)), int(rng.integers(2, 6)))
+    stride = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+    _say("random wide pool", seed, (h, w), win, stride)
+    ref = o.fpool(x, win, stride)
+    dout = dev.empty(ref.size + 32, mis)
+    dev.ffill(-7.0, dout)
+    dev.fpool(dx, dout, h, w, win, stride)
+    got = dout.download()
+    assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
+    assert np.all(got[ref.size:] == -7.0)
+    dx.free(); dout.free()
+
