@@ -35,7 +35,9 @@
 //    window per wave instead of per group, without any group barrier and with
 //    the first output rows computed while the later window rows are still in
 //    flight (105-142 us for 2-8 rows per wave), 16 or more rows per band
-//    (96-115 us); 8 to 12 rows measure the same.
+//    (96-115 us); 8 to 12 rows measured the same then, and with the leaner
+//    row loop 8 rows are 2 % ahead of 12 (87.5 against 89.5 us; 6 rows 91.5,
+//    4 rows 109).
 //  * fpool reads its windows straight from memory: with stride >= window each
 //    input element is used once, and the lanes of a wave walk consecutive
 //    windows, so the lines they touch are consumed completely by that wave.
@@ -64,7 +66,7 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kSegment = 256; // output columns per work-group = lanes
 constexpr int kLine = 32;     // floats per 128-byte line
-constexpr int kConvRows = 12; // output rows per fconv2d work-group
+constexpr int kConvRows = 8;  // output rows per fconv2d work-group
 constexpr int kPoolRows = 2;  // output rows per fpool work-group
 constexpr uint32_t kMaxConvLds = 64 * 1024;
 constexpr int kWaitVmcnt0 = 0x0F70; // s_waitcnt vmcnt(0) with the other counters left alone
