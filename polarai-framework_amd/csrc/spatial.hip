@@ -37,7 +37,16 @@
 //    flight (105-142 us for 2-8 rows per wave), 16 or more rows per band
 //    (96-115 us); 8 to 12 rows measured the same then, and with the leaner
 //    row loop 8 rows are 2 % ahead of 12 (87.5 against 89.5 us; 6 rows 91.5,
-//    4 rows 109).
+//    4 rows 109).  Also slower: no LDS and no barrier at all — a wave walking
+//    down 32-64 rows of 256 columns, each image row fetched once with one
+//    16-byte load per lane, the two columns to the right of a lane's four taken
+//    from the next lane (wave_shl), three rows of partial sums in registers,
+//    three to six rows of fetches in flight with exact vmcnt waits, one 16-byte
+//    store per lane and row: bit-exact, 20 vector instructions per output, and
+//    118-180 us.  Its fetches alone take 48 us and its stores alone 68-80 us
+//    (a plain fill of that size takes 38), and the two add up instead of
+//    overlapping: vmcnt counts loads and stores in order, so a wave that waits
+//    for a fetch also waits for every store it issued before it.
 //  * fpool reads its windows straight from memory: with stride >= window each
 //    input element is used once, and the lanes of a wave walk consecutive
 //    windows, so the lines they touch are consumed completely by that wave.
