@@ -260,8 +260,8 @@ int launchWaves(polar_hip_device* dev, SmallKArgs p, uint32_t groupsPerCu) {
 }
 
 // Sixteen waves per CU either way.  Long operands (from 32768 rows or columns)
-// take them as two groups of eight, each loading the short operand once for
-// two turns: 65536 x 33 x 127 18.0 -> 16.7-17.1 us, 33 x 65536 x 127 16.5 ->
+// take them as two groups of eight, which halves the number of times the short
+// operand is loaded: 65536 x 33 x 127 18.0 -> 16.7-17.1 us, 33 x 65536 x 127 16.5 ->
 // 15.3-15.8 us.  Shorter ones keep four groups of four (8192 x 128 x 128: 15.8
 // against 17.9 us with eight-wave groups).
 template <int TS, bool TA, bool TB, bool TALL>
