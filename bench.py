@@ -46,6 +46,7 @@ SWEEP = ["fadd", "fmul", "fdivide", "fsigmoid", "fcopy", "ffill"]
 # cannot be measured from inside this process, so they are read from the table
 # that summarises those runs; an operation whose kernels the table does not
 # hold reports null.
+LIB_PROBES = os.path.join(ROOT, "bench_probes", "libpolar_hip_probes.so")  # built by bench_probes/Makefile
 TRAFFIC_TABLE = os.path.join(ROOT, "profiles", "bench_kernels_pmc_traffic.md")
 TRAFFIC_KERNELS = {  # operation -> name fragments of the kernels one call launches
     "fadd": ["<AddOp,"], "fmul": ["<MulOp,"], "fdivide": ["<DivOp,"], "fsigmoid": ["<SigmoidOp,"],
@@ -417,7 +418,6 @@ def bench_ceilings(args, n):
     for streams of reads and writes in the ratios the builtins have, and for the
     reads and writes of a tiled transpose of the benchmark's matrix."""
     import ctypes as C
-    from polarai_framework_amd import LIB_PROBES
     lib = C.CDLL(LIB_PROBES)
     reps, warm = max(10, args.steps), max(2, args.warmup)
     us = (C.c_float * reps)()

@@ -26,6 +26,5 @@ REPO_ROOT = os.path.dirname(PACKAGE_DIR)
 
 LIB_DEVICE = os.path.join(PACKAGE_DIR, "libpolar_hip.so")
 LIB_PLUGIN = os.path.join(PACKAGE_DIR, "libpolar_rt_hip.so")
-LIB_PROBES = os.path.join(PACKAGE_DIR, "libpolar_hip_probes.so")  # memory-pattern probes for bench.py
 LIB_HARNESS = os.path.join(PACKAGE_DIR, "libpolar_harness.so")
 TOOL_LSPOLAR = os.path.join(PACKAGE_DIR, "lspolar_hip")  # lists a plugin's devices (the framework's lspolar)

@@ -30,8 +30,8 @@ def test_device_library_exports_every_declared_symbol():
 
 
 def test_probe_library_exports_what_the_benchmark_calls():
-    from polarai_framework_amd import LIB_PROBES
-    lib = C.CDLL(LIB_PROBES)
+    import bench
+    lib = C.CDLL(bench.LIB_PROBES)
     for name in ("polar_probe_streams", "polar_probe_read", "polar_probe_transpose_pattern"):
         assert hasattr(lib, name), name
 
