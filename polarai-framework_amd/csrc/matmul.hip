@@ -580,6 +580,8 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   // short contraction, one long and one short output dimension: streamed in one
   // shot per block (matmul_small_k.hip)
   const MatmulCall call{a, b, c, p.M, p.N, p.K, ta, tb, epilogue, bias, scaleAcc, scaleBias};
+  if (forced.config < 0 && rowsMatmulApplies(call, dev->info.compute_units)) return launchRowsMatmul(dev, call);
+  if (forced.config < 0 && panelMatmulApplies(call, dev->info.compute_units)) return launchPanelMatmul(dev, call);
   if (forced.config < 0 && smallKMatmulApplies(call)) return launchSmallKMatmul(dev, call);
   const MatmulPlan plan =
       forced.config < 0 ? planMatmul(p.M, p.N, p.K, dev->info.compute_units) : forced;

@@ -47,4 +47,16 @@ struct MatmulCall {
 bool smallKMatmulApplies(const MatmulCall& call);
 int launchSmallKMatmul(polar_hip_device* dev, const MatmulCall& call);
 
+// matmul_panel.hip: the same kind of product when the long dimension gives every
+// SIMD of the GPU (computeUnits x 4) a panel of 64 rows or columns of its own.
+// A subset of what smallKMatmulApplies accepts.
+bool panelMatmulApplies(const MatmulCall& call, int computeUnits);
+int launchPanelMatmul(polar_hip_device* dev, const MatmulCall& call);
+
+// matmul_rows.hip: the same again for a long M with A stored row by row, whose
+// rows are fetched as the contiguous memory they are.  A subset of what
+// smallKMatmulApplies accepts (looks at the alignment of call.A).
+bool rowsMatmulApplies(const MatmulCall& call, int computeUnits);
+int launchRowsMatmul(polar_hip_device* dev, const MatmulCall& call);
+
 } // namespace polar_hip_detail

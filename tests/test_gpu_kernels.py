@@ -296,6 +296,50 @@ def test_matmul_short_contraction_tall_and_wide(dev, ta, tb, mnk):
         o.set_threads(1)
 
 
+# One long and one short output dimension with the long one at least 3/4 x 256 x
+# the number of CUs: the kernels that give every SIMD a panel of its own
+# (matmul_panel.hip; matmul_rows.hip when A is stored row by row and aligned).
+LONG_PANEL_SHAPES = [(65536, 33, 127), (65521, 33, 127), (65553, 127, 33), (33, 65536, 127), (65537, 33, 127),
+                     (33, 65541, 127), (65599, 64, 128), (49152, 1, 4), (1, 49153, 5), (70001, 17, 63), (16, 70003, 64),
+                     (66000, 128, 64), (128, 66001, 33), (65536, 48, 100), (48, 65538, 16), (65536, 65, 17),
+                     (100000, 5, 97), (65567, 17, 5), (70000, 128, 16), (65536, 100, 65), (65536, 15, 113)]
+
+
+@pytest.mark.parametrize("misalign", [0, 1])
+@pytest.mark.parametrize("ta", [False, True])
+@pytest.mark.parametrize("tb", [False, True])
+@pytest.mark.parametrize("mnk", LONG_PANEL_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_short_contraction_long_panels(dev, ta, tb, mnk, misalign):
+    """Integer data (exact in any summation order, so a wrong index shows as a
+    wrong value) with line-aligned and with misaligned operands, a guard region
+    on both sides of C; then random data against the oracle."""
+    m, n, k = mnk
+    _say("long-panel matmul", ta, tb, mnk, misalign)
+    rng = np.random.default_rng(m * 13 + n * 1019 + k + 2 * ta + tb)
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    o.set_threads(o.hw_threads())
+    try:
+        a = rng.integers(-4, 5, sa).astype(np.float32)
+        b = rng.integers(-4, 5, sb).astype(np.float32)
+        da, db = dev.array(a, misalign), dev.array(b, misalign)
+        whole = dev.empty(m * n + 128, 0)
+        dev.ffill(-7.0, whole, m * n + 128)
+        dc = type(whole)(dev, m * n, whole.ptr, (64 + misalign) * 4)   # C inside the guarded block
+        dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+        got = whole.download()
+        lo = 64 + misalign
+        assert np.array_equal(got[lo:lo + m * n].reshape(m, n), o.fmatmul(ta, tb, a, b))
+        assert np.all(got[:lo] == -7.0) and np.all(got[lo + m * n:] == -7.0)   # nothing written outside C
+        for t in (da, db, whole):
+            t.free()
+        if misalign == 0:
+            a, b = parity.normal(rng, sa), parity.normal(rng, sb)
+            got = _matmul_device(dev, ta, tb, a, b, m, n, k)
+            assert parity.frobenius_rel_error(got, o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+    finally:
+        o.set_threads(1)
+
+
 NARROW_SHAPES = [(256, 10, 784), (784, 10, 256), (10, 256, 784), (16, 1000, 333), (1000, 16, 16), (64, 1, 5000),
                  (65, 3, 4096), (70, 9, 4097), (5000, 7, 129), (8, 70000, 40), (70000, 5, 200), (300, 16, 17)]
 
