@@ -82,15 +82,19 @@ __device__ __forceinline__ v4f loadUnaligned(const float* p) {
 // 16-byte words.
 constexpr uint32_t panelTileWords(int ts, int groups) { return uint32_t(groups) * ts * 256; }
 
-// TS blocks of 16 cover the short dimension, GROUPS groups of 16 cover K.
-// TALL: M is the long dimension (B is the short operand); otherwise N is.
-template <int TS, int GROUPS, bool TA, bool TB, bool TALL>
+// TS blocks of 16 of the short dimension go through the matrix instruction,
+// GROUPS groups of 16 cover K.  TALL: M is the long dimension (B is the short
+// operand); otherwise N is.  XS: the short dimension is 16 TS + 1, and its last
+// row or column is a dot product on the vector ALUs (33 as three blocks would
+// spend a third of the matrix instructions on 15 rows of padding); otherwise
+// it is at most 16 TS.
+template <int TS, int GROUPS, bool TA, bool TB, bool TALL, bool XS>
 __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   constexpr bool kShortKContig = TALL ? TB : !TA;
   constexpr bool kLongKContig = TALL ? !TA : TB;
   // loads of the short operand per lane: all of it in one go (at most 8192 values)
-  constexpr int SU = TS * GROUPS < 32 ? TS * GROUPS : 32;
+  constexpr int SU = (TS * 16 + (XS ? 1 : 0)) * GROUPS * 16 < 8192 ? ((TS * 16 + (XS ? 1 : 0)) * GROUPS * 16 + kThreads - 1) / kThreads : 32;
   // groups of k whose loads are in flight ahead of the matrix instructions
 #ifndef PANEL_AHEAD
 #define PANEL_AHEAD 4
@@ -169,8 +173,12 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
   // the words of a group and block of 16 x are in lane order.  Element (x, k)
   // with x = 16 j + fx and k = 16 g + r goes to word ((g TS + j) 64 + 16 fk + fx),
   // component c, where r = 4 fk + c (long operand read along k) or r = 4 c + fk.
+  // The extra row or column follows the blocks, 16 values per group, in the
+  // order the lanes multiply them (lane group fk: words 16 g + 4 fk .. + 3).
+  constexpr uint32_t kBlockWords = panelTileWords(TS, GROUPS);
   auto tileAt = [&](uint32_t x, uint32_t k) -> uint32_t {
     const uint32_t r = k % 16;
+    if (XS && x == TS * 16) return kBlockWords + k / 16 * 16 + (kLongKContig ? r : 4 * (r % 4) + r / 4);
     const uint32_t kLane = kLongKContig ? r / 4 : r % 4, c = kLongKContig ? r % 4 : r / 4;
     return (((k / 16) * TS + x / 16) * 64 + kLane * 16 + x % 16) * 4 + c;
   };
@@ -193,7 +201,7 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
       }
     }
     // k in [K, k4) is multiplied (whole groups only), so it holds zeros
-    const uint32_t padK = p.k4 - p.K, xPadded = TS * 16;
+    const uint32_t padK = p.k4 - p.K, xPadded = TS * 16 + (XS ? 1 : 0);
     for (uint32_t e = t; e < padK * xPadded; e += kThreads) lds[tileAt(e % xPadded, p.K + e / xPadded)] = 0.0f;
   }
   __syncthreads();
@@ -240,6 +248,7 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
   v4f frag[2][TS];
 #pragma unroll
   for (int j = 0; j < TS; ++j) frag[0][j] = tile[j * 64];
+  float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // XS: the lane's share of the extra row or column, per block
 #pragma unroll
   for (int g = 0; g < GROUPS; ++g) {
     if (16u * g < p.K) {
@@ -254,7 +263,13 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
       }
       __builtin_amdgcn_sched_barrier(0);
       settle(g);
+      v4f ax = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (XS) ax = *reinterpret_cast<const v4f*>(lds + kBlockWords + 16 * g + 4 * fk);
       auto step = [&](int c) {
+        if constexpr (XS) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) part[i] = __builtin_fmaf(kLongKContig ? buf[g][i][c] : buf[g][c][i], ax[c], part[i]);
+        }
 #pragma unroll
         for (int j = 0; j < TS; ++j) {
 #pragma unroll
@@ -283,6 +298,17 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
   // 5. store.  Accumulator layout: register r of lane l is row 4*(l/16) + r,
   // column l%16 of the 16 x 16 block.
   const uint32_t q = lane / 16;
+  float extra[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  if constexpr (XS) {
+    // the four lanes that hold the same four values of the long dimension (one
+    // per fk) add their shares, in a fixed order
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float p0 = __shfl(part[i], fx), p1 = __shfl(part[i], fx + 16), p2 = __shfl(part[i], fx + 32),
+                  p3 = __shfl(part[i], fx + 48);
+      extra[i] = ((p0 + p1) + p2) + p3;
+    }
+  }
   if constexpr (TALL) {
     // block i, row index m = 4q + r of the block  ->  row x0 + 4m + i of C
     float* const stage = lds + p.shortWords + wave * p.stageWords;
@@ -293,13 +319,25 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const uint32_t local = 4 * (4 * q + r) + i, col = j * 16 + fx;
-          if (col < p.N) {
+          if (XS || col < p.N) {
             float v = acc[i][j][r];
             if (p.epilogue != kEpiNone && x0 + local < longDim)
               v = applyEpilogue(p.epilogue, v, p.bias, p.scaleAcc, p.scaleBias, size_t(x0 + local) * p.N + col);
             stage[local * p.N + col] = v;
           }
         }
+    if constexpr (XS) {
+      // lanes 0..15 hold the extra column of rows x0 + 4 fx + i
+      if (fk == 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float v = extra[i];
+          if (p.epilogue != kEpiNone && x0 + 4 * fx + i < longDim)
+            v = applyEpilogue(p.epilogue, v, p.bias, p.scaleAcc, p.scaleBias, size_t(x0 + 4 * fx + i) * p.N + TS * 16);
+          stage[(4 * fx + i) * p.N + TS * 16] = v;
+        }
+      }
+    }
     // the wave's own writes, read back by other lanes of the same wave: LDS
     // serves a wave's accesses in order
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -331,13 +369,16 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
     const uint32_t col = x0 + 4 * fx;
     const bool whole = col + 4 <= p.N;
 #pragma unroll
-    for (int j = 0; j < TS; ++j)
+    for (int j = 0; j < TS + (XS ? 1 : 0); ++j)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const uint32_t row = j * 16 + 4 * q + r;
-        if (row < p.M) {
+        // the extra row is held by lanes 0..15, all four columns in one lane
+        if (j == TS && r > 0) continue;
+        const uint32_t row = j == TS ? TS * 16 : j * 16 + 4 * q + r;
+        if (j == TS ? fk == 0 : row < p.M) {
           const size_t idx = size_t(row) * p.N + col;
-          v4f v = {acc[0][j][r], acc[1][j][r], acc[2][j][r], acc[3][j][r]};
+          v4f v = {extra[0], extra[1], extra[2], extra[3]};
+          if (j < TS) v = v4f{acc[0][j < TS ? j : 0][r], acc[1][j < TS ? j : 0][r], acc[2][j < TS ? j : 0][r], acc[3][j < TS ? j : 0][r]};
           if (p.epilogue != kEpiNone) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
@@ -355,12 +396,12 @@ __global__ __launch_bounds__(kThreads) void panelKernel(PanelArgs p) {
   }
 }
 
-template <int TS, int GROUPS, bool TA, bool TB, bool TALL>
+template <int TS, int GROUPS, bool TA, bool TB, bool TALL, bool XS>
 int launchPanel(polar_hip_device* dev, PanelArgs p) {
-  p.shortWords = panelTileWords(TS, GROUPS);
+  p.shortWords = panelTileWords(TS, GROUPS) + (XS ? GROUPS * 16 : 0);
   p.stageWords = TALL ? (kSpan * p.N + 3) / 4 * 4 : 0;
   const uint32_t bytes = (p.shortWords + kWaves * p.stageWords) * sizeof(float);
-  auto kernel = panelKernel<TS, GROUPS, TA, TB, TALL>;
+  auto kernel = panelKernel<TS, GROUPS, TA, TB, TALL, XS>;
   // more dynamic LDS than the default limit has to be asked for, once per
   // kernel and device (asking twice is harmless)
   static std::atomic<uint64_t> raised{0};
@@ -376,18 +417,30 @@ int launchPanel(polar_hip_device* dev, PanelArgs p) {
   return POLAR_HIP_OK;
 }
 
+template <int TS, int GROUPS, bool TALL, bool XS>
+int launchStored(polar_hip_device* dev, const PanelArgs& p, bool ta, bool tb) {
+  if (!ta && !tb) return launchPanel<TS, GROUPS, false, false, TALL, XS>(dev, p);
+  if (!ta && tb) return launchPanel<TS, GROUPS, false, true, TALL, XS>(dev, p);
+  if (ta && !tb) return launchPanel<TS, GROUPS, true, false, TALL, XS>(dev, p);
+  return launchPanel<TS, GROUPS, true, true, TALL, XS>(dev, p);
+}
+
 template <int TS, int GROUPS, bool TALL>
 int launchLayouts(polar_hip_device* dev, const PanelArgs& p, bool ta, bool tb) {
-  if (!ta && !tb) return launchPanel<TS, GROUPS, false, false, TALL>(dev, p);
-  if (!ta && tb) return launchPanel<TS, GROUPS, false, true, TALL>(dev, p);
-  if (ta && !tb) return launchPanel<TS, GROUPS, true, false, TALL>(dev, p);
-  return launchPanel<TS, GROUPS, true, true, TALL>(dev, p);
+  if constexpr (TS <= 4) {
+    if ((TALL ? p.N : p.M) == TS * 16 + 1) return launchStored<TS, GROUPS, TALL, true>(dev, p, ta, tb);
+  }
+  return launchStored<TS, GROUPS, TALL, false>(dev, p, ta, tb);
 }
+
+// blocks of 16 of the short dimension that go through the matrix instruction:
+// one row or column beyond up to four whole blocks is computed on the vector ALUs
+uint32_t blocksFor(uint32_t n) { return n > 16 && n <= 65 && n % 16 == 1 ? n / 16 : (n + 15) / 16; }
 
 template <bool TALL>
 int launchBlocks(polar_hip_device* dev, const PanelArgs& p, bool ta, bool tb, uint32_t shortDim) {
   const bool deep = p.k4 > 64;
-  switch ((shortDim + 15) / 16) {
+  switch (blocksFor(shortDim)) {
   case 1: return deep ? launchLayouts<1, 8, TALL>(dev, p, ta, tb) : launchLayouts<1, 4, TALL>(dev, p, ta, tb);
   case 2: return deep ? launchLayouts<2, 8, TALL>(dev, p, ta, tb) : launchLayouts<2, 4, TALL>(dev, p, ta, tb);
   case 3: return deep ? launchLayouts<3, 8, TALL>(dev, p, ta, tb) : launchLayouts<3, 4, TALL>(dev, p, ta, tb);
@@ -413,14 +466,14 @@ bool panelMatmulApplies(const MatmulCall& c, int computeUnits) {
   const bool wide = c.M <= kShortMax && c.N >= longMin;
   if (!tall && !wide) return false;
   const uint32_t shortDim = tall ? c.N : c.M;
-  const uint32_t blocks = (shortDim + 15) / 16, k4 = (c.K + 15) / 16 * 16;
+  const uint32_t blocks = blocksFor(shortDim), k4 = (c.K + 15) / 16 * 16;
   if (blocks > 4 && k4 > 64) return false;
   if (shortDim * c.K > kShortValuesMax) return false;
   if (uint64_t(tall ? c.M : c.N) * c.K * sizeof(float) >= (1ull << 32)) return false; // 32-bit load offsets
   // LDS: the short operand's tile (either orientation) and, for a tall C, the staging areas
   const uint32_t tileWords = panelTileWords(int(blocks), k4 > 64 ? 8 : 4);
   const uint32_t stage = tall ? kWaves * (kSpan * c.N + 4) : 0;
-  return (tileWords + stage) * sizeof(float) <= kMaxLds;
+  return (tileWords + 128 + stage) * sizeof(float) <= kMaxLds;
 }
 
 int launchPanelMatmul(polar_hip_device* dev, const MatmulCall& c) {

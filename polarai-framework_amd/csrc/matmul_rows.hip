@@ -61,11 +61,15 @@ struct RowsArgs {
   float scaleAcc, scaleBias;
 };
 
-// TS blocks of 16 cover N; GROUPS = ceil(K / 16) exactly.  TB: B is stored [N x K].
-template <int TS, int GROUPS, bool TB>
+// TS blocks of 16 columns go through the matrix instruction; GROUPS = ceil(K / 16)
+// exactly.  TB: B is stored [N x K].  XCOL: N = 16 TS + 1, and the one column
+// beyond the blocks is a dot product on the vector ALUs (33 columns as three
+// blocks would spend a third of the matrix instructions on 15 columns of
+// padding); otherwise N <= 16 TS.
+template <int TS, int GROUPS, bool TB, bool XCOL>
 __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  constexpr int SU = (TS * 16 * GROUPS * 16 + kThreads - 1) / kThreads;  // loads of B per lane
+  constexpr int SU = ((TS * 16 + (XCOL ? 1 : 0)) * GROUPS * 16 + kThreads - 1) / kThreads;  // loads of B per lane
   constexpr int LOADS = 2 * GROUPS;  // 16-byte loads of A per lane: 32 rows x at most 16 GROUPS floats
 
   const int t = threadIdx.x, lane = t % 64;
@@ -108,7 +112,10 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
   // 3. B into LDS in the order the matrix instructions want it: element (n, k)
   // with n = 16 j + fx, k = 16 g + 4 fk + c goes to 16-byte word
   // ((g TS + j) 64 + 16 fk + fx), component c.
+  // The extra column's values follow the blocks in the order of k.
+  constexpr uint32_t kBlockWords = uint32_t(GROUPS) * TS * 256;
   auto tileAt = [&](uint32_t n, uint32_t k) -> uint32_t {
+    if (XCOL && n == TS * 16) return kBlockWords + k;
     return (((k / 16) * TS + n / 16) * 64 + (k % 16) / 4 * 16 + n % 16) * 4 + k % 4;
   };
   {
@@ -130,7 +137,7 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
       }
     }
     // k in [K, 16 GROUPS) is multiplied, so it holds zeros
-    const uint32_t padK = GROUPS * 16 - p.K, nPadded = TS * 16;
+    const uint32_t padK = GROUPS * 16 - p.K, nPadded = TS * 16 + (XCOL ? 1 : 0);
     for (uint32_t e = t; e < padK * nPadded; e += kThreads) lds[tileAt(e % nPadded, p.K + e / nPadded)] = 0.0f;
   }
   __syncthreads();
@@ -147,6 +154,11 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
     for (int g = 0; g < GROUPS; ++g)
 #pragma unroll
       for (int j = 0; j < TS; ++j) bq[g][j] = tile[(g * TS + j) * 64];
+  }
+  v4f bx[XCOL ? GROUPS : 1];  // the extra column: the lane's four k of every group
+  if constexpr (XCOL) {
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) bx[g] = *reinterpret_cast<const v4f*>(lds + kBlockWords + 16 * g + 4 * fk);
   }
 
   // 5. block by block: rows into LDS, multiply, rows of C out
@@ -172,10 +184,11 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // LDS serves a wave's accesses in order
   };
 
-  auto multiply = [&](int b, v4f (&acc)[TS]) {
+  auto multiply = [&](int b, v4f (&acc)[TS], float& extra) {
     const float* const mine = area + (16 * b + fx) * p.K + 4 * fk;  // row 16 b + fx, k = 4 fk
 #pragma unroll
     for (int j = 0; j < TS; ++j) acc[j] = v4f{0.f, 0.f, 0.f, 0.f};
+    float part = 0.0f;
     v4f af[2];
     af[0] = *reinterpret_cast<const v4f __attribute__((aligned(4)))*>(mine);
 #pragma unroll
@@ -192,6 +205,16 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
       for (int c = 0; c < 4; ++c)
 #pragma unroll
         for (int j = 0; j < TS; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[c], bq[g][j][c], acc[j], 0, 0, 0);
+      if constexpr (XCOL) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) part = __builtin_fmaf(a[c], bx[g][c], part);
+      }
+    }
+    if constexpr (XCOL) {
+      // the four lanes that hold row fx (one per fk) add their parts, in a fixed order
+      const float p1 = __shfl(part, fx + 16), p2 = __shfl(part, fx + 32), p3 = __shfl(part, fx + 48);
+      const float p0 = __shfl(part, fx);
+      extra = ((p0 + p1) + p2) + p3;
     }
   };
 
@@ -199,7 +222,7 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
   // when they fit there (N <= K), behind the wave's rows of A otherwise -- and
   // leave as one contiguous piece.  Accumulator layout: register r of lane l is
   // row 4 (l / 16) + r, column l % 16.
-  auto storeBlock = [&](int b, const v4f (&acc)[TS]) {
+  auto storeBlock = [&](int b, const v4f (&acc)[TS], float extra) {
     float* const stage = p.N <= p.K ? area + 16 * b * p.K : area + LOADS * 256;
     const uint32_t blockRows = rows - 16 * b < 16 ? rows - 16 * b : 16;
     // no branch per element (with two waves per SIMD a branch still costs the
@@ -213,10 +236,17 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const uint32_t local = 4 * q + r, col = j * 16 + fx;
-          float* const to = (j < TS - 1 || col < p.N) ? stage + local * p.N + col : spare;
+          float* const to = (XCOL || j < TS - 1 || col < p.N) ? stage + local * p.N + col : spare;
           *to = value(j, r, local, col);
         }
     };
+    if constexpr (XCOL) {
+      // lanes 0..15 hold the extra column of rows 0..15 of the block
+      float v = extra;
+      if (p.epilogue != kEpiNone && fx < blockRows)
+        v = applyEpilogue(p.epilogue, v, p.bias, p.scaleAcc, p.scaleBias, size_t(x0 + 16 * b + fx) * p.N + TS * 16);
+      *(fk == 0 ? stage + fx * p.N + TS * 16 : spare) = v;
+    }
     if (p.epilogue == kEpiNone) {
       put([&](int j, int r, uint32_t, uint32_t) { return acc[j][r]; });
     } else {
@@ -256,18 +286,23 @@ __global__ __launch_bounds__(kThreads) void rowsKernel(RowsArgs p) {
   // the wait for those loads would otherwise also wait for the stores issued
   // in between (loads and stores complete in one order).
   v4f acc0[TS], acc1[TS];
+  float extra0 = 0.0f, extra1 = 0.0f;
   placeRows(0);
-  multiply(0, acc0);
+  multiply(0, acc0, extra0);
   const bool second = rows > 16;
   if (second) placeRows(1);
-  storeBlock(0, acc0);
+  storeBlock(0, acc0, extra0);
   if (second) {
-    multiply(1, acc1);
-    storeBlock(1, acc1);
+    multiply(1, acc1, extra1);
+    storeBlock(1, acc1, extra1);
   }
 }
 
 uint32_t roundUp4(uint32_t v) { return (v + 3) / 4 * 4; }
+
+// blocks of 16 columns that go through the matrix instruction: one column
+// beyond a whole number of blocks is computed on the vector ALUs instead
+uint32_t blocksFor(uint32_t n) { return n > 16 && n % 16 == 1 ? n / 16 : (n + 15) / 16; }
 
 // a wave's area: what its loads of A bring (32 rows, rounded up to whole load
 // instructions of 64 x 16 bytes), behind that (when a block's rows of C do not
@@ -278,12 +313,12 @@ uint32_t areaWordsFor(uint32_t n, uint32_t k) {
   return 2 * groups * 256 + (n <= k ? 0 : roundUp4(16 * n)) + 4;
 }
 
-template <int TS, int GROUPS, bool TB>
+template <int TS, int GROUPS, bool TB, bool XCOL>
 int launchRows(polar_hip_device* dev, RowsArgs p) {
-  p.tileWords = uint32_t(GROUPS) * TS * 256;
+  p.tileWords = uint32_t(GROUPS) * TS * 256 + (XCOL ? GROUPS * 16 : 0);
   p.areaWords = areaWordsFor(p.N, p.K);
   const uint32_t bytes = (p.tileWords + kWaves * p.areaWords) * sizeof(float);
-  auto kernel = rowsKernel<TS, GROUPS, TB>;
+  auto kernel = rowsKernel<TS, GROUPS, TB, XCOL>;
   // more dynamic LDS than the default limit has to be asked for, once per
   // kernel and device (asking twice is harmless)
   static std::atomic<uint64_t> raised{0};
@@ -300,7 +335,9 @@ int launchRows(polar_hip_device* dev, RowsArgs p) {
 
 template <int TS, int GROUPS>
 int launchStored(polar_hip_device* dev, const RowsArgs& p, bool tb) {
-  return tb ? launchRows<TS, GROUPS, true>(dev, p) : launchRows<TS, GROUPS, false>(dev, p);
+  if (p.N == TS * 16 + 1)
+    return tb ? launchRows<TS, GROUPS, true, true>(dev, p) : launchRows<TS, GROUPS, false, true>(dev, p);
+  return tb ? launchRows<TS, GROUPS, true, false>(dev, p) : launchRows<TS, GROUPS, false, false>(dev, p);
 }
 
 // TS x GROUPS 16-byte words of B per lane: at most 32
@@ -331,10 +368,10 @@ namespace polar_hip_detail {
 bool rowsMatmulApplies(const MatmulCall& c, int computeUnits) {
   if (c.transA || c.K < 4 || c.K > 128 || c.N > 128) return false;
   if (c.M < kGroupRows * uint32_t(computeUnits) * 3 / 4) return false;  // most CUs get a group of waves
-  const uint32_t blocks = (c.N + 15) / 16, groups = (c.K + 15) / 16;
+  const uint32_t blocks = blocksFor(c.N), groups = (c.K + 15) / 16;
   if (blocks * groups > 32) return false;  // B must fit the registers
   if ((reinterpret_cast<uintptr_t>(c.A) & 15u) != 0) return false;
-  const uint32_t words = groups * blocks * 256 + kWaves * areaWordsFor(c.N, c.K);
+  const uint32_t words = groups * blocks * 256 + groups * 16 + kWaves * areaWordsFor(c.N, c.K);
   return words * sizeof(float) <= kMaxLds;
 }
 
@@ -353,7 +390,7 @@ int launchRowsMatmul(polar_hip_device* dev, const MatmulCall& c) {
   p.scaleBias = c.scaleBias;
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   const uint32_t groups = p.k4 / 16;
-  switch ((c.N + 15) / 16) {
+  switch (blocksFor(c.N)) {
   case 1: return launchGroups<1>(dev, p, c.transB, groups);
   case 2: return launchGroups<2>(dev, p, c.transB, groups);
   case 3: return launchGroups<3>(dev, p, c.transB, groups);
