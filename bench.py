@@ -269,7 +269,58 @@ def main():
 
     if dev is not None:
         dev.close()
+    summary = summarise_into_roofline(result)
     print(json.dumps(result), flush=True)
+    if summary:
+        log(summary)  # last line of the run: the whole metric at a glance
+
+
+RAGGED_PROBES = {  # ragged matmul entry -> the memory-pattern probe that moves the same operands
+    "fmatmul_f_f 65536x127x33 as (M,K,N)": "65536 rows of 127 floats in, 65536 rows of 33 floats out",
+    "fmatmul_f_f 65536x127x33 as (M,N,K)": "65536 rows of 33 floats in, 65536 rows of 127 floats out",
+    "fmatmul_f_f 33x65536x127 as (M,N,K)": "127 rows of 65536 floats in, 33 rows of 65536 floats out",
+}
+
+
+def summarise_into_roofline(result):
+    """The metric has two halves (elementwise GB/s, fp32 matmul GFLOP/s) and the
+    configurations name a transpose and ragged matmuls: their roofline fractions
+    go into `roofline` beside the sweep's dominant kernel, so that one object
+    holds all of them.  Returns a one-line summary."""
+    roof = result["roofline"]
+    parts = [f"sweep {result['value']:.0f} GB/s ({roof['kernel']} {roof['frac']:.3f} of HBM peak)"]
+    mm = result.get("matmul")
+    if mm:
+        variants = mm["variants"].values()
+        roof["matmul"] = {"bound": "mfma", "workload": mm["workload"], "achieved": mm["roofline"]["achieved"],
+                          "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": mm["roofline"]["frac"],
+                          "worst_variant_frac": mm["roofline"]["worst_variant_frac"],
+                          "after_idle_frac": round(float(np.mean([v["isolated_frac_mfma_fp32_peak"] for v in variants])), 4),
+                          "launch_us": round(float(np.mean([v["ms"] for v in variants])) * 1e3, 1),
+                          "launches_before_timing": MM_WARM_LAUNCHES, "traffic": mm["roofline"]["traffic"]}
+        parts.append(f"matmul 4096^3 {roof['matmul']['achieved']:.1f} TFLOP/s ({roof['matmul']['frac']:.3f} of fp32 MFMA "
+                     f"peak settled, {roof['matmul']['after_idle_frac']:.3f} after idle)")
+    tr = result.get("transpose")
+    if tr:
+        roof["transpose"] = dict(tr["roofline"], workload=tr["workload"], launch_us=round(tr["ms"] * 1e3, 1))
+        parts.append(f"transpose {tr['roofline']['frac']:.3f} of HBM peak")
+    ragged = result.get("ragged")
+    if ragged:
+        probes = result.get("ceilings", {}).get("ragged_matmul_pattern", {})
+        entries = {k: v for k, v in ragged.items() if k.startswith("fmatmul")}
+        for name, v in entries.items():
+            probe = probes.get(RAGGED_PROBES.get(name, ""))
+            if probe:
+                v["pattern_probe_us"] = probe["us"]
+                v["first_kernel_vs_probe"] = round(v["first_kernel_us"] / probe["us"], 3)
+        worst = min(entries, key=lambda k: entries[k]["frac_hbm_peak"])
+        roof["ragged_matmul"] = {k: {"frac_hbm": v["frac_hbm_peak"], "us": v["us"],
+                                     "first_kernel_vs_probe": v.get("first_kernel_vs_probe")} for k, v in entries.items()}
+        roof["ragged_worst"] = {"entry": worst, "frac_hbm": entries[worst]["frac_hbm_peak"], "us": entries[worst]["us"],
+                                "buffers_rotated": True}
+        parts.append(f"ragged matmuls {min(v['frac_hbm_peak'] for v in entries.values()):.3f}-"
+                     f"{max(v['frac_hbm_peak'] for v in entries.values()):.3f} of HBM peak on compulsory bytes")
+    return "summary: " + "; ".join(parts)
 
 
 def time_kernel(dev, fn, warmup, reps):
@@ -433,6 +484,8 @@ def bench_ceilings(args, n):
     lib.polar_probe_read.argtypes = [C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_float)]
     lib.polar_probe_transpose_pattern.argtypes = [C.c_uint32, C.c_uint32, C.c_int, C.c_int, C.c_int, C.c_int,
                                                   C.c_int, C.POINTER(C.c_float)]
+    lib.polar_probe_panels.argtypes = [C.c_int, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_int, C.c_int,
+                                       C.POINTER(C.c_float)]
     out = {"note": "probe kernels, not builtins: same bytes and pattern, no work; back-to-back launches, "
                    f"{ROTATE} buffer sets in rotation", "streams": {}, "read_only": {}, "transpose_pattern": {}}
     for reads, like in ((0, "ffill"), (1, "fcopy frelu fsigmoid fconv2d"), (2, "fadd fmul fdivide flogloss"),
@@ -478,6 +531,22 @@ def bench_ceilings(args, n):
                 f"{100 * gbs / HBM_PEAK_GBS:5.1f}%")
     best = max(out["transpose_pattern"].values(), key=lambda v: v["GB/s"])
     out["transpose_pattern"]["best_GB/s"] = best["GB/s"]
+    # the ragged matmuls' memory patterns: rows of the long operand in, rows of C out, no arithmetic
+    out["ragged_matmul_pattern"] = {}
+    for label, wide, long_dim, in_short, out_short in (
+            ("65536 rows of 127 floats in, 65536 rows of 33 floats out", 0, 65536, 127, 33),
+            ("65536 rows of 33 floats in, 65536 rows of 127 floats out", 0, 65536, 33, 127),
+            ("127 rows of 65536 floats in, 33 rows of 65536 floats out", 1, 65536, 127, 33)):
+        nbytes = 4 * long_dim * (in_short + out_short)
+        psets = int(RAGGED_ROTATE_BYTES // nbytes) + 1
+        status = lib.polar_probe_panels(wide, long_dim, in_short, out_short, psets, max(warm, psets), reps, us)
+        if status != 0:
+            raise RuntimeError(f"polar_probe_panels failed with hipError {status}")
+        t = float(np.mean(list(us)))
+        gbs = nbytes / (t * 1e-6) / 1e9
+        out["ragged_matmul_pattern"][label] = {"us": round(t, 2), "GB/s": round(gbs, 1),
+                                               "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "buffer_sets": psets}
+        log(f"probe ragged matmul pattern, {label}: {t:7.1f} us  {gbs:7.1f} GB/s  {100 * gbs / HBM_PEAK_GBS:5.1f}%")
     # the plain copy of the transpose's byte count
     nt = (T_ROWS * T_COLS) // 4 * 4
     t = run(lib.polar_probe_streams, 1, nt, 0, 0, 0)
@@ -544,45 +613,55 @@ def bench_copies(dev):
     return out
 
 
+RAGGED_ROTATE_BYTES = 320 << 20  # bytes a ragged kernel's buffer sets add up to: more than the 256 MB Infinity Cache
+
+
 def bench_ragged(dev, args):
     """The ragged configuration: fadd/fmul on 1 000 003 elements and the two matmul
     shapes 65536x127x33 / 33x65536x127 under both readings of the triple, (M, K, N)
     and (M, N, K).  These are small: both roofline bounds are reported.  `us` is
     the time per call of calls issued back to back (events around each call, so
     kernels that follow a first one are included); `first_kernel_us` is the
-    execution time of the call's first kernel alone."""
-    out = {}
+    execution time of the call's first kernel alone.  Every kernel cycles through
+    as many sets of operands as it takes to exceed the Infinity Cache, so no call
+    finds its operands where the previous call left them."""
+    out = {"buffers_rotated": True, "rotated_bytes": RAGGED_ROTATE_BYTES}
     n = 1000003
     reps = max(20, args.steps)
     rng = np.random.default_rng(9)
-    a, b = dev.array(rng.random(n, dtype=np.float32)), dev.array(rng.random(n, dtype=np.float32))
-    c = dev.empty(n)
-    for name, fn in (("fadd", lambda i: dev.fadd(a, 1.0, b, 1.0, c)), ("fmul", lambda i: dev.fmul(a, b, c))):
-        ms = time_kernel(dev, fn, args.warmup, reps)
+    sets = RAGGED_ROTATE_BYTES // (12 * n) + 1
+    ha, hb = rng.random(n, dtype=np.float32), rng.random(n, dtype=np.float32)
+    das, dbs = device_copies(dev, dev.array(ha), n, sets), device_copies(dev, dev.array(hb), n, sets)
+    dcs = [dev.empty(n) for _ in range(sets)]
+    for name, fn in (("fadd", lambda i: dev.fadd(das[i % sets], 1.0, dbs[i % sets], 1.0, dcs[i % sets])),
+                     ("fmul", lambda i: dev.fmul(das[i % sets], dbs[i % sets], dcs[i % sets]))):
+        ms = time_kernel(dev, fn, max(args.warmup, sets), max(reps, 2 * sets))
         gbs = 12 * n / (np.mean(ms) * 1e-3) / 1e9
         out[f"{name}_{n}"] = {"us": round(float(np.mean(ms)) * 1e3, 2), "GB/s": round(gbs, 1),
-                              "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+                              "frac_hbm_peak": round(gbs / HBM_PEAK_GBS, 4), "buffer_sets": sets}
         log(f"{name} n={n}: {np.mean(ms) * 1e3:7.1f} us  {gbs:7.1f} GB/s")
-    for t in (a, b, c):
+    for t in das + dbs + dcs:
         t.free()
     for label, (m, nn, k) in (("65536x127x33 as (M,K,N)", (65536, 33, 127)), ("65536x127x33 as (M,N,K)", (65536, 127, 33)),
                               ("33x65536x127 as (M,K,N)", (33, 127, 65536)), ("33x65536x127 as (M,N,K)", (33, 65536, 127))):
-        da = dev.array(rng.standard_normal((m, k), dtype=np.float32))
-        db = dev.array(rng.standard_normal((k, nn), dtype=np.float32))
-        dc = dev.empty(m * nn)
-        call = lambda i: dev.fmatmul(0, 0, da, db, dc, m, nn, k)
-        t = float(np.mean(time_calls(dev, call, max(3, args.warmup), reps))) * 1e-3
-        first = float(np.mean(time_kernel(dev, call, 1, reps))) * 1e-3
         flops, nbytes = 2.0 * m * nn * k, 4.0 * (m * k + k * nn + m * nn)
+        sets = int(RAGGED_ROTATE_BYTES // nbytes) + 1
+        das = device_copies(dev, dev.array(rng.standard_normal((m, k), dtype=np.float32)), m * k, sets)
+        dbs = device_copies(dev, dev.array(rng.standard_normal((k, nn), dtype=np.float32)), k * nn, sets)
+        dcs = [dev.empty(m * nn) for _ in range(sets)]
+        call = lambda i: dev.fmatmul(0, 0, das[i % sets], dbs[i % sets], dcs[i % sets], m, nn, k)
+        t = float(np.mean(time_calls(dev, call, max(3, args.warmup, sets), reps))) * 1e-3
+        first = float(np.mean(time_kernel(dev, call, sets, reps))) * 1e-3
         out[f"fmatmul_f_f {label}"] = {"M": m, "N": nn, "K": k, "us": round(t * 1e6, 2),
                                        "first_kernel_us": round(first * 1e6, 2),
                                        "GFLOP/s": round(flops / t / 1e9, 1),
                                        "frac_mfma_fp32_peak": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
                                        "min_bytes_GB/s": round(nbytes / t / 1e9, 1),
-                                       "frac_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4)}
+                                       "frac_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
+                                       "buffer_sets": sets}
         log(f"fmatmul {label}: {t * 1e6:7.1f} us per call (first kernel {first * 1e6:.1f} us)  "
-            f"{flops / t / 1e12:6.2f} TFLOP/s  {nbytes / t / 1e9:7.1f} GB/s of compulsory traffic")
-        for x in (da, db, dc):
+            f"{flops / t / 1e12:6.2f} TFLOP/s  {nbytes / t / 1e9:7.1f} GB/s of compulsory traffic  ({sets} operand sets)")
+        for x in das + dbs + dcs:
             x.free()
     return out
 
@@ -818,24 +897,17 @@ def cpu_baseline(a, b, den, n):
     o.fmatmul(False, False, ma, mb)
     mm_dt = time.perf_counter() - t0
     log(f"cpu oracle fmatmul_f_f 1024^3, 1 thread: {mm_dt:.2f} s, {2 * k ** 3 / mm_dt / 1e9:.2f} GFLOP/s")
-    # the GPU leg's own matmul, 4096^3, with all host threads: a slab of result
-    # rows sized from a short calibration to about 12 s of work (whole rows of
-    # the 4096 x 4096 x 4096 product, so the operands and strides are the real ones)
+    # the GPU leg's own matmul, the whole 4096^3 product, once, with all host threads
     o.set_threads(cores)
     rng = np.random.default_rng(6)
     big_a = rng.standard_normal((MM, MM), dtype=np.float32)
     big_b = rng.standard_normal((MM, MM), dtype=np.float32)
-    probe_rows = 4 * cores
-    t0 = time.perf_counter()
-    o.fmatmul(False, False, big_a, big_b, rows=(0, probe_rows))
-    per_row = (time.perf_counter() - t0) / probe_rows
-    rows = int(min(MM, max(probe_rows, 12.0 / per_row)))
-    rows -= rows % cores
+    rows = MM
     t0 = time.perf_counter()
     o.fmatmul(False, False, big_a, big_b, rows=(0, rows))
     big_dt = time.perf_counter() - t0
     big_gflops = 2.0 * rows * MM * MM / big_dt / 1e9
-    log(f"cpu oracle fmatmul_f_f {MM}^3, {cores} threads, rows 0..{rows}: {big_dt:.2f} s, {big_gflops:.2f} GFLOP/s")
+    log(f"cpu oracle fmatmul_f_f {MM}^3, {cores} threads, the whole product: {big_dt:.2f} s, {big_gflops:.2f} GFLOP/s")
     return {"value": round(res[cores], 2), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"the full sweep ({n} elements per tensor, same inputs), {cores} host threads, "
                       "mean of 3 passes after one warm-up pass",
@@ -843,8 +915,9 @@ def cpu_baseline(a, b, den, n):
             "matmul_1024_single_thread_GFLOP/s": round(2 * k ** 3 / mm_dt / 1e9, 3),
             "matmul_4096": {"value": round(big_gflops, 3), "unit": "GFLOP/s", "cores": cores, "kind": "port",
                             "seconds": round(big_dt, 2),
-                            "sample": f"result rows 0..{rows} of the {MM}x{MM}x{MM} fmatmul_f_f "
-                                      f"({rows}/{MM} of the product, same operands as the GPU leg), {cores} host threads"}}
+                            "extrapolated": False, "rows": rows,
+                            "sample": f"the whole {MM}x{MM}x{MM} fmatmul_f_f, once (same operands as the GPU leg), "
+                                      f"{cores} host threads"}}
 
 
 if __name__ == "__main__":

@@ -206,6 +206,57 @@ void launchPattern(hipStream_t s, hipEvent_t e0, hipEvent_t e1, const float* in,
 
 } // namespace
 
+// ---- panels: the memory pattern of a short-contraction matmul with one long
+// dimension, without the arithmetic ------------------------------------------
+// tall: `longDim` rows of `inShort` floats in (one contiguous array), `longDim`
+// rows of `outShort` floats out; a wave takes 32 rows: their input as the
+// contiguous piece it is, 16 bytes per lane and load, all loads first; their
+// output likewise.
+__global__ __launch_bounds__(512) void tallPanelsKernel(const float* in, float* out, uint32_t longDim,
+                                                        uint32_t inShort, uint32_t outShort) {
+  const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const uint32_t x0 = blockIdx.x * 256 + wave * 32;
+  if (x0 >= longDim) return;
+  const uint32_t rows = longDim - x0 < 32 ? longDim - x0 : 32;
+  const uint32_t inFloats = rows * inShort, outFloats = rows * outShort;
+  const float* const piece = in + size_t(x0) * inShort;
+  v4f v[16];
+#pragma unroll
+  for (int u = 0; u < 16; ++u) {
+    const uint32_t at = (u * 64 + lane) * 4;
+    v[u] = *reinterpret_cast<const v4f*>(piece + (at + 4 <= inFloats ? at : 0));
+  }
+  v4f acc = v[0];
+#pragma unroll
+  for (int u = 1; u < 16; ++u)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = v[u][c] > acc[c] ? v[u][c] : acc[c];
+  float* const to = out + size_t(x0) * outShort;
+  for (uint32_t at = lane * 4; at + 4 <= outFloats; at += 256) *reinterpret_cast<v4f*>(to + at) = acc;
+}
+// wide: `inShort` rows of `longDim` floats in, `outShort` rows of `longDim`
+// floats out; a wave takes 64 columns, a quarter of it one row per instruction:
+// four rows of 256 bytes per load and per store, all loads first.
+template <int LOADS>
+__global__ __launch_bounds__(256) void widePanelsKernel(const float* in, float* out, uint32_t longDim,
+                                                        uint32_t inShort, uint32_t outShort) {
+  const uint32_t lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const uint32_t x = blockIdx.x * 256 + wave * 64 + 4 * (lane % 16), q = lane / 16;
+  if (x + 4 > longDim) return;
+  v4f v[LOADS];
+#pragma unroll
+  for (int u = 0; u < LOADS; ++u) {
+    const uint32_t k = 4 * u + q;
+    v[u] = *reinterpret_cast<const v4f*>(in + size_t(k < inShort ? k : inShort - 1) * longDim + x);
+  }
+  v4f acc = v[0];
+#pragma unroll
+  for (int u = 1; u < LOADS; ++u)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] = v[u][c] > acc[c] ? v[u][c] : acc[c];
+  for (uint32_t r = q; r < outShort; r += 4) *reinterpret_cast<v4f*>(out + size_t(r) * longDim + x) = acc;
+}
+
 extern "C" {
 
 // `reads` input streams of n floats each combined into one output stream of n
@@ -308,6 +359,44 @@ int polar_probe_transpose_pattern(uint32_t rows, uint32_t cols, int variant, int
     case 4: launchPattern<32, 64, 256>(st.s, e0, e1, in, out, rows, cols, order); break;
     default: launchPattern<128, 64, 512>(st.s, e0, e1, in, out, rows, cols, order); break;
     }
+  });
+}
+
+// The memory pattern of C[long x outShort] = A[long x inShort] * B (wide = 0:
+// rows of inShort floats in, rows of outShort floats out) or of its mirror
+// image C[outShort x long] = A * B[inShort x long] (wide = 1).  inShort <= 128;
+// tall needs 32 * inShort <= 4096, both need the long dimension to be a
+// multiple of 4.  Bytes per launch: 4 long (inShort + outShort).
+int polar_probe_panels(int wide, uint32_t longDim, uint32_t inShort, uint32_t outShort, int sets, int warm,
+                       int reps, float* us) {
+  if (longDim == 0 || longDim % 4 != 0 || inShort == 0 || inShort > 128 || outShort == 0 || outShort > 128 ||
+      sets < 1 || reps < 1)
+    return hipErrorInvalidValue;
+  Buffers mem;
+  Stream st;
+  PROBE_TRY(hipSetDevice(0));
+  PROBE_TRY(st.make());
+  std::vector<float*> ins(sets), outs(sets);
+  for (int k = 0; k < sets; ++k) {
+    PROBE_TRY(mem.add(size_t(longDim) * inShort * 4 + 4096, reinterpret_cast<void**>(&ins[k])));
+    PROBE_TRY(mem.add(size_t(longDim) * outShort * 4 + 4096, reinterpret_cast<void**>(&outs[k])));
+  }
+  const unsigned grid = (longDim + 255) / 256;
+  return timeLaunches(st.s, warm, reps, us, [&](int i, hipEvent_t e0, hipEvent_t e1) {
+    const float* in = ins[i % sets];
+    float* out = outs[i % sets];
+    if (!wide)
+      hipExtLaunchKernelGGL(tallPanelsKernel, dim3(grid), dim3(512), 0, st.s, e0, e1, 0, in, out, longDim, inShort,
+                            outShort);
+    else if (inShort <= 32)
+      hipExtLaunchKernelGGL(widePanelsKernel<8>, dim3(grid), dim3(256), 0, st.s, e0, e1, 0, in, out, longDim,
+                            inShort, outShort);
+    else if (inShort <= 64)
+      hipExtLaunchKernelGGL(widePanelsKernel<16>, dim3(grid), dim3(256), 0, st.s, e0, e1, 0, in, out, longDim,
+                            inShort, outShort);
+    else
+      hipExtLaunchKernelGGL(widePanelsKernel<32>, dim3(grid), dim3(256), 0, st.s, e0, e1, 0, in, out, longDim,
+                            inShort, outShort);
   });
 }
 

@@ -32,7 +32,7 @@ def test_device_library_exports_every_declared_symbol():
 def test_probe_library_exports_what_the_benchmark_calls():
     import bench
     lib = C.CDLL(bench.LIB_PROBES)
-    for name in ("polar_probe_streams", "polar_probe_read", "polar_probe_transpose_pattern"):
+    for name in ("polar_probe_streams", "polar_probe_read", "polar_probe_transpose_pattern", "polar_probe_panels"):
         assert hasattr(lib, name), name
 
 
