@@ -279,6 +279,18 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in,
 int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
                     uint64_t height, uint64_t width, uint64_t window0,
                     uint64_t window1, uint64_t stride0, uint64_t stride1);
+/* Which kernel polar_hip_fpool takes for a call, without running it (the
+ * pooling counterpart of polar_hip_fmatmul_plan; needs no device).
+ * input_aligned: the input pointer is 16-byte aligned.  *kernel: 0 = every tap
+ * read from memory, 1 = non-overlapping 2x2 / 4x4 windows read by vectors,
+ * 2 = the band's input window staged in LDS; then *band_rows output rows per
+ * work-group and *lds_bytes of LDS (either may be null).  No counterpart in the
+ * reference, whose pooling is generated code
+ * (utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:45-82). */
+int polar_hip_fpool_plan(uint64_t height, uint64_t width, uint64_t window0,
+                         uint64_t window1, uint64_t stride0, uint64_t stride1,
+                         int input_aligned, int* kernel, uint32_t* band_rows,
+                         uint32_t* lds_bytes);
 
 /* ---- Extended (fused) builtins -------------------------------------------------
  * The reference's design allows runtimes to offer fused builtins that

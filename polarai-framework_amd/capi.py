@@ -99,6 +99,8 @@ SIGNATURES = {
     "polar_hip_fsoftmax_static": (_i, [_vp, _vp, _vp, _u64]),
     "polar_hip_fconv2d": (_i, [_vp, _vp, _vp, _vp, _u64, _u64, _u64, _u64]),
     "polar_hip_fpool": (_i, [_vp, _vp, _vp, _u64, _u64, _u64, _u64, _u64, _u64]),
+    "polar_hip_fpool_plan": (_i, [_u64, _u64, _u64, _u64, _u64, _u64, _i, C.POINTER(C.c_int), C.POINTER(C.c_uint32),
+                                  C.POINTER(C.c_uint32)]),
     "polar_hip_fmatmul_fsigmoid": (_i, [_vp, _i, _i, _vp, _vp, _vp, _u64, _u64, _u64]),
     "polar_hip_fmatmul_fadd_fsigmoid": (_i, [_vp, _i, _i, _vp, _vp, _f, _vp, _f, _vp, _u64, _u64, _u64]),
     "polar_hip_fsigmoid_flogloss": (_i, [_vp, _vp, _vp, _vp, _u64]),
@@ -129,6 +131,17 @@ def load_library(path=LIB_DEVICE):
 def _check(lib, status):
     if status != 0:
         raise PolarHipError(status, lib.polar_hip_last_error().decode())
+
+
+def fpool_plan(height, width, window, stride, input_aligned=True):
+    """(kernel, band rows, LDS bytes) polar_hip_fpool would use: kernel 0 = taps
+    from memory, 1 = non-overlapping square windows, 2 = window staged in LDS.
+    Needs no GPU."""
+    lib = load_library()
+    kernel, band, lds = _i(0), C.c_uint32(0), C.c_uint32(0)
+    _check(lib, lib.polar_hip_fpool_plan(height, width, window[0], window[1], stride[0], stride[1],
+                                         int(bool(input_aligned)), C.byref(kernel), C.byref(band), C.byref(lds)))
+    return kernel.value, band.value, lds.value
 
 
 def device_count():

@@ -124,28 +124,30 @@ __host__ __device__ constexpr uint32_t convPitch(uint32_t kw, bool vec) {
 }
 
 // LDS reads with the distance from a base address in the instruction (up to 64
-// KB), for unrolled taps.  The compiler does not know what the asm does, so
-// the wait for the data is explicit: ldsReadsDone takes the values as operands,
-// which keeps every use of them behind it.
+// KB), for unrolled taps: the three taps of a row of the 3 x 3 kernel for the
+// lane's four outputs (64 floats apart), twelve reads, and the wait for them,
+// in ONE asm statement.  The compiler does not track what an asm issues, so a
+// read whose wait sat in a later statement would leave registers that look
+// written but are not until then -- nothing would stop a copy or a spill in
+// between from reading them early.  The outputs are early-clobber: the address
+// register is read by all twelve instructions.
 __device__ __forceinline__ uint32_t ldsAddress(const float* p) {
   return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
       (const __attribute__((address_space(3))) float*)(p)));
 }
 template <uint32_t kByteOffset>
-__device__ __forceinline__ float ldsReadAt(uint32_t address) {
-  static_assert(kByteOffset < 65536, "offset field of the LDS read");
-  float v;
-  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(address), "n"(kByteOffset));
-  return v;
-}
-template <int... I, typename F>
-__device__ __forceinline__ void forEachConstant(std::integer_sequence<int, I...>, F f) {
-  (f(std::integral_constant<int, I>{}), ...);
-}
-__device__ __forceinline__ void ldsReadsDone(float (&v)[4][3]) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(v[0][0]), "+v"(v[0][1]), "+v"(v[0][2]), "+v"(v[1][0]), "+v"(v[1][1]), "+v"(v[1][2]),
-                 "+v"(v[2][0]), "+v"(v[2][1]), "+v"(v[2][2]), "+v"(v[3][0]), "+v"(v[3][1]), "+v"(v[3][2]));
+__device__ __forceinline__ void ldsReadTapRow(uint32_t address, float (&v)[4][3]) {
+  static_assert(kByteOffset + 3 * 256 + 8 < 65536, "offset field of the LDS read");
+  asm volatile(
+      "ds_read_b32 %0, %12 offset:%13\n\tds_read_b32 %1, %12 offset:%13+4\n\tds_read_b32 %2, %12 offset:%13+8\n\t"
+      "ds_read_b32 %3, %12 offset:%13+256\n\tds_read_b32 %4, %12 offset:%13+260\n\tds_read_b32 %5, %12 offset:%13+264\n\t"
+      "ds_read_b32 %6, %12 offset:%13+512\n\tds_read_b32 %7, %12 offset:%13+516\n\tds_read_b32 %8, %12 offset:%13+520\n\t"
+      "ds_read_b32 %9, %12 offset:%13+768\n\tds_read_b32 %10, %12 offset:%13+772\n\tds_read_b32 %11, %12 offset:%13+776\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(v[0][0]), "=&v"(v[0][1]), "=&v"(v[0][2]), "=&v"(v[1][0]), "=&v"(v[1][1]), "=&v"(v[1][2]),
+        "=&v"(v[2][0]), "=&v"(v[2][1]), "=&v"(v[2][2]), "=&v"(v[3][0]), "=&v"(v[3][1]), "=&v"(v[3][2])
+      : "v"(address), "n"(kByteOffset)
+      : "memory");
 }
 
 // KH_/KW_ == 0: the kernel size comes from the arguments.  VEC: image rows
@@ -309,15 +311,9 @@ __global__ __launch_bounds__(kSegment) void conv2dKernel(ConvArgs p) {
       constexpr uint32_t P = convPitch(3, VEC);
       const uint32_t at = ldsAddress(win);
       float v[3][4][3];
-      forEachConstant(std::make_integer_sequence<int, 12>{}, [&](auto index) {
-        constexpr int a = decltype(index)::value / 4, j = decltype(index)::value % 4;
-        v[a][j][0] = ldsReadAt<(a * P + 64 * j + 0) * 4>(at);
-        v[a][j][1] = ldsReadAt<(a * P + 64 * j + 1) * 4>(at);
-        v[a][j][2] = ldsReadAt<(a * P + 64 * j + 2) * 4>(at);
-      });
-      ldsReadsDone(v[0]);
-      ldsReadsDone(v[1]);
-      ldsReadsDone(v[2]);
+      ldsReadTapRow<0 * P * 4>(at, v[0]);
+      ldsReadTapRow<1 * P * 4>(at, v[1]);
+      ldsReadTapRow<2 * P * 4>(at, v[2]);
 #pragma unroll
       for (int a = 0; a < 3; ++a)
 #pragma unroll
@@ -591,6 +587,38 @@ __global__ __launch_bounds__(kSegment) void poolStagedKernel(PoolStagedArgs q) {
   }
 }
 
+// Geometry of the staged pooling kernel for one call, or fits = false if a band
+// of one output row does not fit its LDS budget.  All of it in 64 bits: the
+// strides are only bounded by the image (2^31), and a pitch that wrapped in 32
+// bits could pass for one that fits.
+struct StagedPoolPlan {
+  bool fits;
+  uint32_t pitch, lead, bandRows, ldsBytes;
+};
+StagedPoolPlan planStagedPool(const PoolArgs& p, bool vec) {
+  StagedPoolPlan plan{false, 0, 0, 0, 0};
+  uint64_t pitch = uint64_t(kSegment + kLine - 2) * p.stride1 + p.win1, lead = 0;
+  // Image rows that start on 16 bytes: the window is staged by vectors.  Its
+  // first needed column is (256 ct - 31) stride1, the same modulo 4 for every
+  // column tile; the staged window starts that many columns earlier.
+  if (vec) {
+    lead = (4 - (uint64_t(kLine - 1) * p.stride1) % 4) % 4;
+    pitch = (pitch + lead + 3) / 4 * 4;
+  }
+  const uint64_t floats = kMaxPoolLds / sizeof(float);
+  if (pitch > floats) return plan;
+  const uint64_t rowsFit = floats / pitch; // input rows
+  if (rowsFit < p.win0 || uint64_t(p.H) * p.W >= (1ull << 40)) return plan;
+  uint64_t band = (rowsFit - p.win0) / p.stride0 + 1;
+  if (band > kPoolStagedRows) band = kPoolStagedRows;
+  plan.fits = true;
+  plan.pitch = static_cast<uint32_t>(pitch);
+  plan.lead = static_cast<uint32_t>(lead);
+  plan.bandRows = static_cast<uint32_t>(band);
+  plan.ldsBytes = static_cast<uint32_t>(((band - 1) * p.stride0 + p.win0) * pitch * sizeof(float));
+  return plan;
+}
+
 uint32_t phaseOf(const float* out) {
   return static_cast<uint32_t>((reinterpret_cast<uintptr_t>(out) / sizeof(float)) % kLine);
 }
@@ -649,6 +677,41 @@ int polar_hip_fconv2d(polar_hip_device* dev, const float* in, const float* kerne
   return POLAR_HIP_OK;
 }
 
+int polar_hip_fpool_plan(uint64_t height, uint64_t width, uint64_t window0, uint64_t window1,
+                         uint64_t stride0, uint64_t stride1, int input_aligned, int* kernel,
+                         uint32_t* band_rows, uint32_t* lds_bytes) {
+  POLAR_HIP_REQUIRE(kernel != nullptr, "null argument");
+  POLAR_HIP_REQUIRE(window0 >= 1 && window1 >= 1, "empty pooling window");
+  POLAR_HIP_REQUIRE(stride0 >= 1 && stride1 >= 1, "pooling stride must be positive");
+  POLAR_HIP_REQUIRE(height >= window0 && width >= window1, "pooling window larger than the input");
+  POLAR_HIP_REQUIRE(height < (1ull << 31) && width < (1ull << 31), "dimension does not fit 31 bits");
+  PoolArgs p{};
+  p.H = static_cast<uint32_t>(height);
+  p.W = static_cast<uint32_t>(width);
+  p.win0 = static_cast<uint32_t>(window0);
+  p.win1 = static_cast<uint32_t>(window1);
+  p.stride0 = static_cast<uint32_t>(stride0 < height ? stride0 : height);
+  p.stride1 = static_cast<uint32_t>(stride1 < width ? stride1 : width);
+  const bool aligned = input_aligned != 0;
+  auto square = [&](uint32_t w) {
+    return p.win0 == w && p.win1 == w && p.stride0 == w && p.stride1 == w && p.W % w == 0 && aligned;
+  };
+  *kernel = 0;
+  if (band_rows) *band_rows = 0;
+  if (lds_bytes) *lds_bytes = 0;
+  if (square(2) || square(4)) {
+    *kernel = 1;
+    return POLAR_HIP_OK;
+  }
+  const StagedPoolPlan plan = planStagedPool(p, aligned && p.W % 4 == 0);
+  if (plan.fits) {
+    *kernel = 2;
+    if (band_rows) *band_rows = plan.bandRows;
+    if (lds_bytes) *lds_bytes = plan.ldsBytes;
+  }
+  return POLAR_HIP_OK;
+}
+
 int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
                     uint64_t height, uint64_t width, uint64_t window0,
                     uint64_t window1, uint64_t stride0, uint64_t stride1) {
@@ -686,35 +749,23 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
   };
   if (!square(2) && !square(4)) {
     // staged kernel if a band of at least one output row fits the LDS budget
-    PoolStagedArgs q;
-    q.pool = p;
-    q.pitch = (kSegment + kLine - 2) * p.stride1 + p.win1;
-    q.lead = 0;
-    // Image rows that start on 16 bytes: the window is staged by vectors.  Its
-    // first needed column is (256 ct - 31) stride1, the same modulo 4 for every
-    // column tile; the staged window starts that many columns earlier.
     const bool vec = p.W % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0;
-    if (vec) {
-      q.lead = static_cast<uint32_t>((4 - (uint64_t(kLine - 1) * p.stride1) % 4) % 4);
-      q.pitch = (q.pitch + q.lead + 3) / 4 * 4;
-    }
-    const uint64_t floats = kMaxPoolLds / sizeof(float);
-    const uint64_t rowsFit = floats / q.pitch; // input rows
-    if (rowsFit >= p.win0 && uint64_t(p.H) * p.W < (1ull << 40)) {
-      uint64_t band = (rowsFit - p.win0) / p.stride0 + 1;
-      if (band > kPoolStagedRows) band = kPoolStagedRows;
-      q.bandRows = static_cast<uint32_t>(band);
+    const StagedPoolPlan plan = planStagedPool(p, vec);
+    if (plan.fits) {
+      PoolStagedArgs q;
+      q.pool = p;
+      q.pitch = plan.pitch;
+      q.lead = plan.lead;
+      q.bandRows = plan.bandRows;
       const uint64_t stagedTiles = uint64_t(p.colTiles) * ((p.OH + q.bandRows - 1) / q.bandRows);
       POLAR_HIP_REQUIRE(stagedTiles < (1ull << 31) - kXcds, "tensor too large for one launch");
       q.pool.tiles = static_cast<uint32_t>(stagedTiles);
-      const uint32_t ldsBytes = static_cast<uint32_t>(
-          (uint64_t(q.bandRows - 1) * p.stride0 + p.win0) * q.pitch * sizeof(float));
       auto staged = p.win0 == 2 && p.win1 == 2   ? (vec ? poolStagedKernel<2, 2, true> : poolStagedKernel<2, 2, false>)
                     : p.win0 == 3 && p.win1 == 3 ? (vec ? poolStagedKernel<3, 3, true> : poolStagedKernel<3, 3, false>)
                     : p.win0 == 5 && p.win1 == 5 ? (vec ? poolStagedKernel<5, 5, true> : poolStagedKernel<5, 5, false>)
                                                  : (vec ? poolStagedKernel<0, 0, true> : poolStagedKernel<0, 0, false>);
       POLAR_HIP_TRY(launchKernelLds(dev, staged, dim3(static_cast<unsigned>(paddedGrid(stagedTiles))),
-                                    dim3(kSegment), ldsBytes, q));
+                                    dim3(kSegment), plan.ldsBytes, q));
       return POLAR_HIP_OK;
     }
   }

@@ -29,6 +29,23 @@ def test_device_library_exports_every_declared_symbol():
     assert sorted(capi.SIGNATURES) == names  # the binding covers the header exactly
 
 
+def test_pool_plan_stays_off_the_staged_kernel_when_the_stride_overflows_32_bits():
+    """The staged pooling kernel's window pitch is 286 x stride1 + window1 floats:
+    for strides of tens of millions that product wraps in 32 bits and could pass
+    for a pitch that fits LDS.  The planner works in 64 bits."""
+    staged = capi.fpool_plan(8192, 8192, (3, 3), (2, 2))
+    assert staged[0] == 2 and staged[1] >= 1 and 0 < staged[2] <= 24 * 1024
+    assert capi.fpool_plan(8192, 8192, (2, 2), (2, 2))[0] == 1
+    assert capi.fpool_plan(8192, 8192, (2, 2), (2, 2), input_aligned=False)[0] == 2
+    wide = (1 << 31) - 1
+    for stride1 in (15_017_369, 15_017_370, 15_017_372, 30_034_737, 2**24, 2**26 + 5, wide // 2):
+        # 286 * stride1 + 3 is 241, 527, 1099 and 193 modulo 2^32 for the first four
+        kernel, band, lds = capi.fpool_plan(4, wide, (3, 3), (1, stride1))
+        assert (kernel, band, lds) == (0, 0, 0), (stride1, kernel, band, lds)
+    assert capi.fpool_plan(64, 100000, (5, 5), (2, 4))[0] == 2      # five input rows of 1152 floats fit 24 KiB
+    assert capi.fpool_plan(64, 100000, (5, 5), (2, 5))[0] == 0      # of 1436 floats: only four do
+
+
 def test_probe_library_exports_what_the_benchmark_calls():
     import bench
     lib = C.CDLL(bench.LIB_PROBES)
