@@ -81,12 +81,13 @@ struct polar_hip_device {
   void* softmaxScratch = nullptr;
 
   // Workspace of the builtins that run more than one kernel per call (softmax
-  // partial sums, split-K partial products): one block allocated when the
-  // device is opened and sized for the largest request the library makes, so
-  // that a launch neither allocates nor waits.  workspaceMu is held while a
-  // call enqueues the kernels that share it.
+  // partial sums, split-K partial products): one block that grows on demand to
+  // the largest request seen so far (workspaceFor), so that a call whose size
+  // has been seen before neither allocates nor waits.  workspaceMu is held
+  // while a call enqueues the kernels that share it.
   std::mutex workspaceMu;
   void* workspace = nullptr;
+  uint64_t workspaceBytes = 0;
   // Transfers queued directly out of or into blocks of polar_hip_host_alloc are
   // numbered per device handle; directDone is the highest number known to be
   // complete, learnt from whatever the caller waits for anyway (an event
@@ -94,6 +95,9 @@ struct polar_hip_device {
   // events of their own.  `serial` names this handle in the blocks' bookkeeping.
   uint64_t serial = 0;
   std::atomic<uint64_t> directQueued{0}, directDone{0};
+  // threads waiting for this handle's stream on behalf of a host block, outside
+  // the table's mutex; the handle is not destroyed while there are any
+  std::atomic<int> waiters{0};
   void noteDirectDone(uint64_t number) {
     uint64_t seen = directDone.load(std::memory_order_relaxed);
     while (seen < number && !directDone.compare_exchange_weak(seen, number)) {
@@ -119,8 +123,9 @@ int resolveStaticScratch(polar_hip_device* dev); // elementwise.hip
 // The matmul planner never asks for more split-K workspace than this, and the
 // partial sums of a softmax over 2^31 elements take 256 KiB.
 constexpr uint64_t kWorkspaceBytes = 256ull << 20;
-// *area: the device's workspace (kWorkspaceBytes, 256-byte aligned, contents
-// undefined).  Caller holds dev->workspaceMu.  Fails for a larger request.
+// *area: the device's workspace, at least `bytes` long (256-byte aligned,
+// contents undefined), grown if it was smaller.  Caller holds dev->workspaceMu.
+// Fails for a request above kWorkspaceBytes.
 int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area); // runtime.hip
 
 // Every kernel of the library is launched through here.  Normally a plain

@@ -181,12 +181,14 @@ int launchWaves(polar_hip_device* dev, SmallKArgs p, uint32_t groupsPerCu) {
   auto kernel = smallKKernel<TS, TA, TB, TALL, WAVES>;
   // more dynamic LDS than the default limit has to be asked for, once per
   // kernel and device
-  static uint64_t raised = 0;
+  // (asking twice, from two threads at once, is harmless; launching before the
+  // first request has returned is not, so the flag is set after it)
+  static std::atomic<uint64_t> raised{0};
   const uint64_t bit = 1ull << (dev->ordinal & 63);
-  if (bytes > 48 * 1024 && !(raised & bit)) {
+  if (bytes > 48 * 1024 && !(raised.load(std::memory_order_acquire) & bit)) {
     POLAR_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-    raised |= bit;
+    raised.fetch_or(bit, std::memory_order_release);
   }
   // one turn per group up to groupsPerCu groups per CU; beyond that groups take
   // several turns (and load the short operand once for all of them)

@@ -50,10 +50,35 @@ int failHip(hipError_t e, const char* what) {
 
 // ---- workspace ----------------------------------------------------------------
 
+// The block grows on demand, in powers of two from 4 MiB up to kWorkspaceBytes:
+// a handle that never splits a contraction or takes a softmax holds nothing,
+// and one that does holds what its largest call so far needed.  Growing waits
+// for the stream (kernels may still be using the old block) and allocates, so
+// the first call of a new size pays for it once; calls after it neither
+// allocate nor wait.
 int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area) {
   if (bytes > kWorkspaceBytes)
-    return fail(POLAR_HIP_ERR_INVALID, "workspace request of %llu bytes exceeds the %llu the device holds",
+    return fail(POLAR_HIP_ERR_INVALID, "workspace request of %llu bytes exceeds the cap of %llu",
                 static_cast<unsigned long long>(bytes), static_cast<unsigned long long>(kWorkspaceBytes));
+  if (bytes > dev->workspaceBytes) {
+    uint64_t size = 4ull << 20;
+    while (size < bytes) size *= 2;
+    hipError_t e = hipSetDevice(dev->ordinal);
+    if (e != hipSuccess) return failHip(e, "hipSetDevice");
+    if (dev->workspace != nullptr) {
+      e = hipStreamSynchronize(dev->stream);
+      if (e != hipSuccess) return failHip(e, "hipStreamSynchronize (workspace)");
+      (void)hipFree(dev->workspace);
+      dev->workspace = nullptr;
+      dev->workspaceBytes = 0;
+    }
+    e = hipMalloc(&dev->workspace, size);
+    if (e != hipSuccess) {
+      dev->workspace = nullptr;
+      return failHip(e, "hipMalloc (workspace)");
+    }
+    dev->workspaceBytes = size;
+  }
   *area = dev->workspace;
   return POLAR_HIP_OK;
 }
@@ -115,10 +140,6 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
   d->info.pci_bus_id = p.pciBusID;
   d->info.hbm_bytes = p.totalGlobalMem;
   st = resolveStaticScratch(d);
-  if (st == POLAR_HIP_OK) {
-    e = hipMalloc(&d->workspace, polar_hip_detail::kWorkspaceBytes);
-    if (e != hipSuccess) st = failHip(e, "hipMalloc (workspace)");
-  }
   if (st != POLAR_HIP_OK) {
     (void)hipStreamDestroy(d->stream);
     delete d;
@@ -143,6 +164,9 @@ int polar_hip_device_close(polar_hip_device* dev) {
     std::lock_guard<std::mutex> g(g_hostMu);
     g_openDevices.erase(dev->serial);
   }
+  // a thread that found the handle before it left the table may still be waiting
+  // for its stream (waitForBlock, outside the mutex): let it finish
+  while (dev->waiters.load() != 0) std::this_thread::yield();
   for (auto& kv : dev->cached)
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : dev->live) (void)hipFree(kv.first);
@@ -433,45 +457,74 @@ struct HostBlock {
 };
 std::map<uintptr_t, HostBlock> g_hostBlocks; // by base address; g_hostMu
 
-// the block that holds [p, p + bytes), or null; g_hostMu held
-HostBlock* hostBlockOf(const void* p, uint64_t bytes) {
+// the block that holds [p, p + bytes) and its base address, or null; g_hostMu held
+HostBlock* hostBlockOf(const void* p, uint64_t bytes, uintptr_t* base = nullptr) {
   const uintptr_t a = reinterpret_cast<uintptr_t>(p);
   auto it = g_hostBlocks.upper_bound(a);
   if (it == g_hostBlocks.begin()) return nullptr;
   --it;
-  return a + bytes <= it->first + it->second.bytes ? &it->second : nullptr;
+  if (a + bytes > it->first + it->second.bytes) return nullptr;
+  if (base != nullptr) *base = it->first;
+  return &it->second;
 }
 
-// Returns once the latest transfer queued on the block is complete.  Usually
-// that is already known: the caller has waited for an event recorded behind the
-// transfer (every launch of a graph is followed by one), and the device handle
-// has noted how far its stream had got.  Otherwise the whole stream is waited
-// for.  No event per transfer: a recorded event puts a marker packet between
-// the kernels, and waiting for an idle stream costs tens of microseconds.
-// g_hostMu held.
-hipError_t waitForBlock(HostBlock& b) {
-  if (b.number == 0) return hipSuccess;
-  auto it = g_openDevices.find(b.serial);
-  if (it != g_openDevices.end() && it->second->directDone.load() < b.number) {
+// Returns once every transfer that was queued on the block at `base` when the
+// call began is complete.  Usually that is already known: the caller has waited
+// for an event recorded behind the transfer (every launch of a graph is followed
+// by one), and the device handle has noted how far its stream had got.
+// Otherwise the whole stream is waited for.  No event per transfer: a recorded
+// event puts a marker packet between the kernels, and waiting for an idle
+// stream costs tens of microseconds.
+// `lock` holds g_hostMu on entry and on return, but NOT while the stream is
+// waited for: the mutex is process-wide (every copy on every device takes it to
+// look its buffer up), and a stream may be milliseconds long.  The block may
+// have been freed or used again in between, so the caller looks it up afresh;
+// the device handle is kept open by its count of waiters (polar_hip_device_close).
+hipError_t waitForBlock(std::unique_lock<std::mutex>& lock, uintptr_t base) {
+  for (;;) {
+    auto bi = g_hostBlocks.find(base);
+    if (bi == g_hostBlocks.end() || bi->second.number == 0) return hipSuccess;
+    const uint64_t number = bi->second.number, serial = bi->second.serial;
+    auto it = g_openDevices.find(serial);
+    if (it == g_openDevices.end() || it->second->directDone.load() >= number) {
+      bi->second.number = 0;
+      return hipSuccess;
+    }
     polar_hip_device* dev = it->second;
     const uint64_t queued = dev->directQueued.load();
+    dev->waiters.fetch_add(1);
+    lock.unlock();
     const hipError_t e = hipStreamSynchronize(dev->stream);
+    if (e == hipSuccess) dev->noteDirectDone(queued);
+    dev->waiters.fetch_sub(1);
+    lock.lock();
     if (e != hipSuccess) return e;
-    dev->noteDirectDone(queued);
+    // look again: the note may be gone, or name a later transfer of another thread
+    bi = g_hostBlocks.find(base);
+    if (bi == g_hostBlocks.end()) return hipSuccess;
+    if (bi->second.number == number && bi->second.serial == serial) {
+      bi->second.number = 0;
+      return hipSuccess;
+    }
+    if (bi->second.serial == serial) return hipSuccess;  // a later transfer on the stream we drained: not ours to wait for
   }
-  b.number = 0;
-  return hipSuccess;
 }
 
 // Queue a transfer between a host block and device memory on dev's stream and
 // note it on the block.  g_hostMu held.
-hipError_t queueDirect(polar_hip_device* dev, HostBlock& b, void* dst, const void* src, uint64_t bytes,
-                       hipMemcpyKind kind) {
+hipError_t queueDirect(std::unique_lock<std::mutex>& lock, polar_hip_device* dev, uintptr_t base, void* dst,
+                       const void* src, uint64_t bytes, hipMemcpyKind kind, uint64_t* number = nullptr) {
   // another handle's transfer on the block first: one note per block
-  if (b.number != 0 && b.serial != dev->serial) {
-    const hipError_t w = waitForBlock(b);
-    if (w != hipSuccess) return w;
+  {
+    auto bi = g_hostBlocks.find(base);
+    if (bi != g_hostBlocks.end() && bi->second.number != 0 && bi->second.serial != dev->serial) {
+      const hipError_t w = waitForBlock(lock, base);
+      if (w != hipSuccess) return w;
+    }
   }
+  auto found = g_hostBlocks.find(base);
+  if (found == g_hostBlocks.end()) return hipErrorInvalidValue;  // freed by another thread while we waited
+  HostBlock& b = found->second;
   hipError_t e;
   if (bytes < kTwoThreadBytes && ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src)) & 15u) == 0) {
     const uint32_t vectors = static_cast<uint32_t>(bytes / 16), tail = static_cast<uint32_t>(bytes % 16);
@@ -484,6 +537,7 @@ hipError_t queueDirect(polar_hip_device* dev, HostBlock& b, void* dst, const voi
   if (e != hipSuccess) return e;
   b.serial = dev->serial;
   b.number = dev->directQueued.fetch_add(1) + 1; // after the launch: an event stamped with it is behind the transfer
+  if (number != nullptr) *number = b.number;
   return hipSuccess;
 }
 } // namespace
@@ -505,12 +559,21 @@ int polar_hip_host_alloc(polar_hip_device* dev, uint64_t bytes, void** ptr) {
 int polar_hip_host_free(void* ptr) {
   if (ptr == nullptr) return POLAR_HIP_OK;
   {
-    std::lock_guard<std::mutex> g(g_hostMu);
-    auto it = g_hostBlocks.find(reinterpret_cast<uintptr_t>(ptr));
-    if (it == g_hostBlocks.end())
+    std::unique_lock<std::mutex> g(g_hostMu);
+    const uintptr_t base = reinterpret_cast<uintptr_t>(ptr);
+    if (g_hostBlocks.find(base) == g_hostBlocks.end())
       return fail(POLAR_HIP_ERR_INVALID, "polar_hip_host_free: %p is not a block of polar_hip_host_alloc", ptr);
-    POLAR_HIP_TRY(waitForBlock(it->second));
-    g_hostBlocks.erase(it);
+    // until nothing is outstanding: another thread may queue while the mutex is released
+    for (;;) {
+      POLAR_HIP_TRY(waitForBlock(g, base));
+      auto it = g_hostBlocks.find(base);
+      if (it == g_hostBlocks.end())
+        return fail(POLAR_HIP_ERR_INVALID, "polar_hip_host_free: %p was freed by another thread", ptr);
+      if (it->second.number == 0) {
+        g_hostBlocks.erase(it);
+        break;
+      }
+    }
   }
   POLAR_HIP_TRY(hipHostFree(ptr));
   return POLAR_HIP_OK;
@@ -518,11 +581,11 @@ int polar_hip_host_free(void* ptr) {
 
 int polar_hip_host_quiesce(void* ptr) {
   if (ptr == nullptr) return POLAR_HIP_OK;
-  std::lock_guard<std::mutex> g(g_hostMu);
-  HostBlock* b = hostBlockOf(ptr, 1);
-  if (b == nullptr)
+  std::unique_lock<std::mutex> g(g_hostMu);
+  uintptr_t base = 0;
+  if (hostBlockOf(ptr, 1, &base) == nullptr)
     return fail(POLAR_HIP_ERR_INVALID, "polar_hip_host_quiesce: %p is not inside a block of polar_hip_host_alloc", ptr);
-  POLAR_HIP_TRY(waitForBlock(*b));
+  POLAR_HIP_TRY(waitForBlock(g, base));
   return POLAR_HIP_OK;
 }
 
@@ -535,9 +598,10 @@ int polar_hip_copy_to_device(polar_hip_device* dev, void* dst_device,
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   {
     // source inside a block of polar_hip_host_alloc: no staging
-    std::lock_guard<std::mutex> g(g_hostMu);
-    if (HostBlock* b = hostBlockOf(src_host, bytes)) {
-      POLAR_HIP_TRY(queueDirect(dev, *b, dst_device, src_host, bytes, hipMemcpyHostToDevice));
+    std::unique_lock<std::mutex> g(g_hostMu);
+    uintptr_t base = 0;
+    if (hostBlockOf(src_host, bytes, &base) != nullptr) {
+      POLAR_HIP_TRY(queueDirect(g, dev, base, dst_device, src_host, bytes, hipMemcpyHostToDevice));
       return POLAR_HIP_OK;
     }
   }
@@ -631,11 +695,10 @@ int polar_hip_copy_to_host(polar_hip_device* dev, void* dst_host,
     // of the block are ahead of the new one on its stream)
     uint64_t number = 0;
     {
-      std::lock_guard<std::mutex> g(g_hostMu);
-      if (HostBlock* b = hostBlockOf(dst_host, bytes)) {
-        POLAR_HIP_TRY(queueDirect(dev, *b, dst_host, src_device, bytes, hipMemcpyDeviceToHost));
-        number = b->number;
-      }
+      std::unique_lock<std::mutex> g(g_hostMu);
+      uintptr_t base = 0;
+      if (hostBlockOf(dst_host, bytes, &base) != nullptr)
+        POLAR_HIP_TRY(queueDirect(g, dev, base, dst_host, src_device, bytes, hipMemcpyDeviceToHost, &number));
     }
     if (number != 0) {
       // wait outside the table's lock (a large read-back takes milliseconds);
