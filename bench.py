@@ -114,6 +114,9 @@ def main():
                     help="skip the ragged-shape leg (keeps a profile to one problem size per kernel)")
     ap.add_argument("--no-probes", action="store_true",
                     help="skip the memory-pattern probes (pattern ceilings measured beside the builtins)")
+    ap.add_argument("--legs", default="transpose,matmul,next,ragged,mid,copies",
+                    help="which legs follow the sweep (comma-separated, of transpose, matmul, next, ragged, mid, "
+                         "copies): a counter run names the ones whose kernels it is after")
     ap.add_argument("--no-graphs", action="store_true",
                     help="skip the model-graph legs (keeps a profile to one problem size per kernel)")
     args = ap.parse_args()
@@ -248,14 +251,24 @@ def main():
     for buf in list(outs.values()) + [dden]:
         buf.free()
 
-    if not args.no_matmul:
+    legs = set(args.legs.split(",")) if not args.no_matmul else set()
+    unknown = legs - {"transpose", "matmul", "next", "ragged", "mid", "copies", ""}
+    if unknown:
+        sys.exit(f"bench.py: unknown leg(s) {sorted(unknown)}")
+    if args.no_ragged:
+        legs -= {"ragged", "mid", "copies"}
+    if "transpose" in legs:
         result["transpose"] = bench_transpose(dev, args)
+    if "matmul" in legs:
         result["matmul"] = bench_matmul(dev, args)
+    if "next" in legs:
         result["next_builtins"] = bench_next_builtins(dev, da, n, args)
-        if not args.no_ragged:
-            result["ragged"] = bench_ragged(dev, args)
-            result["matmul_mid_size"] = bench_matmul_mid(dev, args)
-            result["copies"] = bench_copies(dev)
+    if "ragged" in legs:
+        result["ragged"] = bench_ragged(dev, args)
+    if "mid" in legs:
+        result["matmul_mid_size"] = bench_matmul_mid(dev, args)
+    if "copies" in legs:
+        result["copies"] = bench_copies(dev)
     da.free(); db.free()
     dev.close()
     dev = None
