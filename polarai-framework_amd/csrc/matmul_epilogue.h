@@ -59,4 +59,11 @@ int launchPanelMatmul(polar_hip_device* dev, const MatmulCall& call);
 bool rowsMatmulApplies(const MatmulCall& call, int computeUnits);
 int launchRowsMatmul(polar_hip_device* dev, const MatmulCall& call);
 
+
+// matmul_long_k.hip: a long contraction with a result of at most 33 x 128, both
+// operands as stored: one slice of K per CU, partial results added in a second
+// kernel.
+bool longKMatmulApplies(const MatmulCall& call);
+int launchLongKMatmul(polar_hip_device* dev, const MatmulCall& call);
+
 } // namespace polar_hip_detail

@@ -340,6 +340,46 @@ def test_matmul_short_contraction_long_panels(dev, ta, tb, mnk, misalign):
         o.set_threads(1)
 
 
+# A long contraction with a result of at most 33 x 128, operands as stored: one
+# slice of K per CU and a second kernel that adds the partial results
+# (matmul_long_k.hip).  K not a multiple of 4, 16 or 64 exercises the clamped
+# loads at the end of both operands.
+LONG_K_SHAPES = [(33, 127, 65536), (33, 127, 65537), (33, 128, 70001), (32, 100, 16384), (17, 64, 20000), (16, 4, 16385),
+                 (1, 65, 33333), (33, 5, 65539), (9, 127, 100003), (16, 4, 16386), (31, 33, 262144)]
+
+
+@pytest.mark.parametrize("misalign", [0, 1])
+@pytest.mark.parametrize("mnk", LONG_K_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_matmul_long_contraction_small_result(dev, mnk, misalign):
+    m, n, k = mnk
+    _say("long-k matmul", mnk, misalign)
+    assert dev.fmatmul_plan(m, n, k)[0] == -1
+    rng = np.random.default_rng(m * 17 + n * 1021 + k)
+    o.set_threads(o.hw_threads())
+    try:
+        a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+        da, db = dev.array(a, misalign), dev.array(b, misalign)
+        whole = dev.empty(m * n + 128, 0)
+        dev.ffill(-7.0, whole, m * n + 128)
+        lo = 64 + misalign
+        dc = type(whole)(dev, m * n, whole.ptr, lo * 4)
+        dev.fmatmul(False, False, da, db, dc, m, n, k)
+        got = whole.download()
+        assert np.array_equal(got[lo:lo + m * n].reshape(m, n), o.fmatmul(False, False, a, b))
+        assert np.all(got[:lo] == -7.0) and np.all(got[lo + m * n:] == -7.0)
+        first = got.copy()
+        dev.fmatmul(False, False, da, db, dc, m, n, k)
+        assert np.array_equal(whole.download(), first)                      # repeatable
+        for t in (da, db, whole):
+            t.free()
+        a, b = parity.normal(rng, (m, k)), parity.normal(rng, (k, n))
+        got = _matmul_device(dev, False, False, a, b, m, n, k)
+        assert parity.frobenius_rel_error(got, o.fmatmul(False, False, a, b)) <= parity.MATMUL_FRO_REL
+    finally:
+        o.set_threads(1)
+
+
 NARROW_SHAPES = [(256, 10, 784), (784, 10, 256), (10, 256, 784), (16, 1000, 333), (1000, 16, 16), (64, 1, 5000),
                  (65, 3, 4096), (70, 9, 4097), (5000, 7, 129), (8, 70000, 40), (70000, 5, 200), (300, 16, 17)]
 
