@@ -284,7 +284,9 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
  * input_aligned: the input pointer is 16-byte aligned.  *kernel: 0 = every tap
  * read from memory, 1 = non-overlapping 2x2 / 4x4 windows read by vectors,
  * 2 = the band's input window staged in LDS; then *band_rows output rows per
- * work-group and *lds_bytes of LDS (either may be null).  No counterpart in the
+ * work-group and *lds_bytes of LDS (either may be null), 3 = overlapping square
+ * windows of 4 or 5 at stride 1 or 2 over rows that start on 16 bytes: waves
+ * march down strips of *band_rows output rows, row folds kept in registers.  No counterpart in the
  * reference, whose pooling is generated code
  * (utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:45-82). */
 int polar_hip_fpool_plan(uint64_t height, uint64_t width, uint64_t window0,

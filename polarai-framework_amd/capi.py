@@ -135,8 +135,8 @@ def _check(lib, status):
 
 def fpool_plan(height, width, window, stride, input_aligned=True):
     """(kernel, band rows, LDS bytes) polar_hip_fpool would use: kernel 0 = taps
-    from memory, 1 = non-overlapping square windows, 2 = window staged in LDS.
-    Needs no GPU."""
+    from memory, 1 = non-overlapping square windows, 2 = window staged in LDS,
+    3 = waves marching down strips (square windows of 4 and 5).  Needs no GPU."""
     lib = load_library()
     kernel, band, lds = _i(0), C.c_uint32(0), C.c_uint32(0)
     _check(lib, lib.polar_hip_fpool_plan(height, width, window[0], window[1], stride[0], stride[1],

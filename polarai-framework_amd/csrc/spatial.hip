@@ -587,6 +587,247 @@ __global__ __launch_bounds__(kSegment) void poolStagedKernel(PoolStagedArgs q) {
   }
 }
 
+// Overlapping square windows of 2..5 at stride 1 or 2 over rows that start on 16
+// bytes: a wave marches down a strip of the image.  Every lane holds STRIDE
+// 16-byte vectors of each input row (kMarchAhead rows in flight), takes the
+// columns its windows reach beyond a vector from the lane that holds the next
+// one, and folds the row's taps of each of its four outputs into one value; the
+// last WIN rows of those values stay in registers and are folded again when a
+// window is complete.  Each input element is loaded once per strip (the WIN -
+// stride rows two bands share, twice) and every tap costs a compare and a
+// select instead of an LDS read.
+//
+// Stores decide the rest.  A row of the wave's outputs leaves through 1 KB of
+// LDS, so that it can be cut where the 128-byte lines of the output are, not
+// where the lanes' columns are: the wave whose nominal piece of the row (220
+// columns) holds the start of a line stores that line, whole.  A wave therefore
+// computes 252 (stride 2: 254) columns and stores up to 251 of them, the pieces
+// of neighbouring waves overlapping by what that takes; only the two ends of an
+// output row are stored as parts of lines.  (With every lane storing its own
+// four columns, a row left as 1008-byte pieces that shared a line at either
+// end: 127 us for 3 x 3 windows at stride 1 over 8192^2, 48 us of it loads.)
+//
+// The order of the comparisons is the reference's: rows in ascending order,
+// columns in ascending order within a row, strictly greater replaces.  Folding
+// each row first and the rows' results afterwards picks the same element as
+// one pass over the window does -- the first of the largest -- so the result is
+// the same bit pattern even where +0 and -0 meet, and NaNs are skipped as
+// there, because every fold starts from the floor value, not from an element.
+constexpr uint32_t kMarchChunk = 220;   // output columns between the first columns of neighbouring waves
+// Rows a wave has in flight, and waves a launch aims for (the bands get shorter
+// to reach it, down to kMarchMinBand output rows).  8192^2, stride 1: 125 us
+// with 8192 waves, 104 with 16384, 96 with 65536 or more (six rows in flight;
+// eight: 1 us less; twelve: more registers, slower again) -- short bands keep
+// the rows that many waves read and write at one time close together in
+// memory.  Stride 2 has half the stores and prefers long bands, which read
+// fewer rows twice: 5 x 5, 66 us with 8192 waves, 67-70 with 16384-65536.
+template <int STRIDE> constexpr int kMarchAhead = STRIDE == 1 ? 8 : 6;
+constexpr uint32_t marchWaves(uint32_t stride) { return stride == 1 ? 65536 : 8192; }
+constexpr uint32_t kMarchMinBand = 8;   // output rows per wave, at least
+
+struct PoolMarchArgs {
+  PoolArgs pool;
+  uint32_t vecsPerRow;  // W / 4
+  uint32_t wavesAcross; // ceil(OW / 220)
+  uint32_t bandRows;    // output rows per wave
+};
+
+typedef float v2f __attribute__((ext_vector_type(2)));  // (LDS only)
+
+template <int WIN, int STRIDE>
+__global__ __launch_bounds__(64) void poolMarchKernel(PoolMarchArgs q) {
+  constexpr int VPL = STRIDE;                                  // vectors of a row per lane
+  constexpr int NOUT = 4 / STRIDE;                             // outputs per vector and output row
+  constexpr int REACH = (NOUT - 1) * STRIDE + WIN;             // columns the windows of a vector span
+  constexpr int HALO = REACH > 4 ? REACH - 4 : 0;              // of them, in the next vector
+  constexpr int D = kMarchAhead<STRIDE>;
+  static_assert(4 % STRIDE == 0 && HALO <= 4, "a vector's windows end within the next vector");
+  static_assert(kMarchChunk * STRIDE % 4 == 0, "every wave starts on a vector");
+  static_assert(kMarchChunk + 31 <= uint32_t(NOUT) * (64 * VPL - 1), "what a wave may have to store, it computes");
+  __shared__ __attribute__((aligned(16))) float stage[64 * VPL * NOUT];
+  const PoolArgs& p = q.pool;
+  uint32_t task;
+  if (!tileOfGroup(p.tiles, &task)) return;
+  const uint32_t lane = threadIdx.x;
+  const uint32_t across = task % q.wavesAcross, band = task / q.wavesAcross;
+  const uint32_t y0 = band * q.bandRows;
+  const uint32_t outRows = p.OH - y0 < q.bandRows ? p.OH - y0 : q.bandRows;
+  const uint32_t inRows = (outRows - 1) * STRIDE + WIN;
+  const uint32_t firstColumn = across * kMarchChunk;  // of the wave's outputs
+  // the lane's vectors of a row: 64 j + lane behind the wave's first; beyond the
+  // row, some valid address (no output that is stored depends on it)
+  const v4f* src[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    uint32_t vec = firstColumn * STRIDE / 4 + 64 * j + lane;
+    if (vec >= q.vecsPerRow) vec = q.vecsPerRow - 1;
+    src[j] = reinterpret_cast<const v4f*>(p.in + uint64_t(y0) * STRIDE * p.W) + vec;
+  }
+  const uint64_t pitchVecs = q.vecsPerRow;
+  // the output row being completed: where the wave's first column is, in floats from `out`
+  uint64_t flat = uint64_t(y0) * p.OW + firstColumn;
+  const uint64_t outFloats = reinterpret_cast<uintptr_t>(p.out) / sizeof(float);
+  const uint32_t columnsLeft = p.OW - firstColumn;  // of the row, from the wave's first
+
+  const uint32_t lastRow = inRows - 1;
+  v4f ahead[D][VPL];
+#pragma unroll
+  for (int d = 0; d < D; ++d)
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) ahead[d][j] = src[j][(uint32_t(d) < inRows ? d : lastRow) * pitchVecs];
+  float h[WIN][VPL][NOUT];  // the row folds of the last WIN rows, oldest first
+#pragma unroll
+  for (int a = 0; a < WIN; ++a)
+#pragma unroll
+    for (int j = 0; j < VPL; ++j)
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) h[a][j][i] = -10e5f;
+
+  // one more input row: its folds enter the ring
+  auto fold = [&](const v4f (&own)[VPL]) {
+#pragma unroll
+    for (int a = 0; a + 1 < WIN; ++a)
+#pragma unroll
+      for (int j = 0; j < VPL; ++j)
+#pragma unroll
+        for (int i = 0; i < NOUT; ++i) h[a][j][i] = h[a + 1][j][i];
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      float c[4 + HALO];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) c[e] = own[j][e];
+      // the next vector of the row is the next lane's, and for lane 63 lane 0's
+      // next one (the wave's last vector has none: its outputs are never stored)
+#pragma unroll
+      for (int e = 0; e < HALO; ++e) {
+        const float mine = (j + 1 < VPL && lane == 0) ? own[j + 1 < VPL ? j + 1 : j][e] : own[j][e];
+        c[4 + e] = __shfl(mine, (lane + 1) & 63);
+      }
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) {
+        // utils/dialects/lib/PolarGraph/kernels/Pool2DOp.cpp:50-52,74-76: starts
+        // at -10e5, strict ordered greater-than
+        float best = -10e5f;
+#pragma unroll
+        for (int b = 0; b < WIN; ++b) best = c[i * STRIDE + b] > best ? c[i * STRIDE + b] : best;
+        h[WIN - 1][j][i] = best;
+      }
+    }
+  };
+  // the ring holds a complete window: one output row
+  auto emit = [&]() {
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) {
+      float o[NOUT];
+#pragma unroll
+      for (int i = 0; i < NOUT; ++i) {
+        float best = -10e5f;
+#pragma unroll
+        for (int a = 0; a < WIN; ++a) best = h[a][j][i] > best ? h[a][j][i] : best;
+        o[i] = best;
+      }
+      // column NOUT (64 j + lane) + i of the wave
+      if constexpr (NOUT == 4)
+        *reinterpret_cast<v4f*>(stage + 4 * (64 * j + lane)) = v4f{o[0], o[1], o[2], o[3]};
+      else
+        *reinterpret_cast<v2f*>(stage + 2 * (64 * j + lane)) = v2f{o[0], o[1]};
+    }
+    // The wave stores columns [from, to) of its own: from the first line that
+    // starts in its piece (the row's first wave: from the row's start) up to
+    // the first line that starts in the next wave's piece, or the row's end.
+    const uint32_t phase = uint32_t(outFloats + flat) & 31u;  // of the wave's first column within its line
+    const uint32_t from = across == 0 ? 0 : (32 - phase) & 31u;
+    uint32_t to = kMarchChunk + ((32 - ((phase + kMarchChunk) & 31u)) & 31u);
+    if (to > columnsLeft) to = columnsLeft;
+    // in pieces of 16 bytes, one per lane; only a row's first and last can be
+    // partly outside
+    const int32_t first = int32_t(from) - int32_t((phase + from) & 3u) + 4 * int32_t(lane);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the row is in LDS (a wave's LDS accesses are served in order)
+    float v[4];
+    bool inside[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int32_t at = first + e;
+      inside[e] = at >= int32_t(from) && at < int32_t(to);
+      v[e] = stage[inside[e] ? at : 0];
+    }
+    float* const dst = p.out + flat + first;  // (only dereferenced where inside)
+    // (stores the compiler does not count: its waits for the rows in flight stay exact)
+    if (inside[0] && inside[3]) {
+      streamStore(v4f{v[0], v[1], v[2], v[3]}, reinterpret_cast<v4f*>(dst));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (inside[e]) streamStore(v[e], dst + e);
+    }
+    flat += p.OW;
+  };
+
+  // the first WIN - 1 rows complete no window
+  constexpr int P = WIN - 1;
+  static_assert(P < D && D % STRIDE == 0, "the slots and the output rows repeat with the unrolled loop");
+#pragma unroll
+  for (int a = 0; a < P; ++a) {
+    fold(ahead[a]);
+#pragma unroll
+    for (int j = 0; j < VPL; ++j) ahead[a][j] = src[j][(uint32_t(a + D) < inRows ? a + D : lastRow) * pitchVecs];
+  }
+  // From here on row P + n completes a window when n is a multiple of the
+  // stride, and sits in slot (P + n) % D.  While 2 D rows remain, every fetch
+  // of the loop is of a row of the band: no conditions, so the waits can be
+  // exact.
+  uint32_t row = P;
+  for (; row + 2 * D <= inRows; row += D) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) {
+      const int slot = (P + d) % D;
+      fold(ahead[slot]);
+#pragma unroll
+      for (int j = 0; j < VPL; ++j) ahead[slot][j] = src[j][uint64_t(row + d + D) * pitchVecs];
+      if (d % STRIDE == 0) emit();
+    }
+  }
+  // the last rows (fewer than 2 D)
+#pragma unroll
+  for (int d = 0; d < 2 * D; ++d) {
+    if (row + d < inRows) {  // (uniform)
+      const int slot = (P + d) % D;
+      fold(ahead[slot]);
+      if (row + d + D < inRows) {
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) ahead[slot][j] = src[j][uint64_t(row + d + D) * pitchVecs];
+      }
+      if (d % STRIDE == 0) emit();
+    }
+  }
+}
+
+// Whether a call goes to the marching kernel, and its geometry
+struct MarchPoolPlan {
+  bool fits;
+  uint32_t vecsPerRow, wavesAcross, bandRows;
+  uint64_t tasks;
+};
+MarchPoolPlan planMarchPool(const PoolArgs& p, bool vec) {
+  MarchPoolPlan plan{false, 0, 0, 0, 0};
+  const bool square = p.win0 == p.win1 && p.stride0 == p.stride1;
+  // Windows of 2 and 3 stay with the staged kernel, which reads fewer input
+  // columns twice (8192^2, kernel time, staged / marching: 3 x 3 stride 1 90 /
+  // 96 us, stride 2 56 / 66, 2 x 2 stride 1 88 / 95; but 4 x 4 stride 1 138 /
+  // 101, stride 2 68 / 66, 5 x 5 stride 1 180 / 108, stride 2 99 / 66).
+  if (!vec || !square || p.win0 < 4 || p.win0 > 5 || p.stride0 < 1 || p.stride0 > 2) return plan;
+  plan.vecsPerRow = p.W / 4;
+  plan.wavesAcross = (p.OW + kMarchChunk - 1) / kMarchChunk;
+  const uint32_t bandsWanted = marchWaves(p.stride0) / plan.wavesAcross > 0 ? marchWaves(p.stride0) / plan.wavesAcross : 1;
+  uint32_t band = (p.OH + bandsWanted - 1) / bandsWanted;
+  if (band < kMarchMinBand) band = kMarchMinBand;
+  if (band > p.OH) band = p.OH;
+  plan.bandRows = band;
+  plan.tasks = uint64_t(plan.wavesAcross) * ((p.OH + band - 1) / band);
+  plan.fits = plan.tasks < (1ull << 31) - kXcds;
+  return plan;
+}
+
 // Geometry of the staged pooling kernel for one call, or fits = false if a band
 // of one output row does not fit its LDS budget.  All of it in 64 bits: the
 // strides are only bounded by the image (2^31), and a pitch that wrapped in 32
@@ -692,6 +933,8 @@ int polar_hip_fpool_plan(uint64_t height, uint64_t width, uint64_t window0, uint
   p.win1 = static_cast<uint32_t>(window1);
   p.stride0 = static_cast<uint32_t>(stride0 < height ? stride0 : height);
   p.stride1 = static_cast<uint32_t>(stride1 < width ? stride1 : width);
+  p.OH = (p.H - p.win0) / p.stride0 + 1;
+  p.OW = (p.W - p.win1) / p.stride1 + 1;
   const bool aligned = input_aligned != 0;
   auto square = [&](uint32_t w) {
     return p.win0 == w && p.win1 == w && p.stride0 == w && p.stride1 == w && p.W % w == 0 && aligned;
@@ -701,6 +944,12 @@ int polar_hip_fpool_plan(uint64_t height, uint64_t width, uint64_t window0, uint
   if (lds_bytes) *lds_bytes = 0;
   if (square(2) || square(4)) {
     *kernel = 1;
+    return POLAR_HIP_OK;
+  }
+  const MarchPoolPlan march = planMarchPool(p, aligned && p.W % 4 == 0);
+  if (march.fits) {
+    *kernel = 3;
+    if (band_rows) *band_rows = march.bandRows;
     return POLAR_HIP_OK;
   }
   const StagedPoolPlan plan = planStagedPool(p, aligned && p.W % 4 == 0);
@@ -750,6 +999,25 @@ int polar_hip_fpool(polar_hip_device* dev, const float* in, float* out,
   if (!square(2) && !square(4)) {
     // staged kernel if a band of at least one output row fits the LDS budget
     const bool vec = p.W % 4 == 0 && reinterpret_cast<uintptr_t>(in) % 16 == 0;
+    const MarchPoolPlan march = planMarchPool(p, vec);
+    if (march.fits) {
+      PoolMarchArgs q;
+      q.pool = p;
+      q.pool.tiles = static_cast<uint32_t>(march.tasks);
+      q.vecsPerRow = march.vecsPerRow;
+      q.wavesAcross = march.wavesAcross;
+      q.bandRows = march.bandRows;
+      void (*marching)(PoolMarchArgs) = nullptr;
+      switch (p.win0 * 10 + p.stride0) {
+      case 41: marching = poolMarchKernel<4, 1>; break;
+      case 42: marching = poolMarchKernel<4, 2>; break;
+      case 51: marching = poolMarchKernel<5, 1>; break;
+      case 52: marching = poolMarchKernel<5, 2>; break;
+      }
+      POLAR_HIP_REQUIRE(marching != nullptr, "no marching kernel for this window");
+      POLAR_HIP_TRY(launchKernel(dev, marching, dim3(static_cast<unsigned>(paddedGrid(march.tasks))), dim3(64), q));
+      return POLAR_HIP_OK;
+    }
     const StagedPoolPlan plan = planStagedPool(p, vec);
     if (plan.fits) {
       PoolStagedArgs q;

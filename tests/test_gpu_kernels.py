@@ -765,7 +765,14 @@ POOL_CASES = [((4, 4), (2, 2), (2, 2)), ((100, 257), (2, 2), (2, 2)), ((101, 333
               ((300, 1200), (3, 3), (1, 1)), ((133, 777), (2, 2), (1, 1)), ((200, 2100), (3, 3), (2, 2)),
               ((97, 1500), (5, 5), (2, 2)), ((64, 900), (2, 3), (4, 5)), ((41, 290), (3, 3), (3, 3)),
               ((40, 258), (7, 2), (1, 1)), ((300, 40), (3, 5), (2, 1)), ((13, 4000), (13, 1), (1, 2)),
-              ((120, 600), (30, 30), (5, 5)), ((60, 700), (3, 200), (2, 100))]
+              ((120, 600), (30, 30), (5, 5)), ((60, 700), (3, 200), (2, 100)),
+              # the marching kernel (square windows of 4 and 5, stride 1 and 2, widths that are multiples of 4):
+              # several waves across and bands down, an output width one past a wave's 220 columns, a ragged
+              # last band, images smaller than one wave or one band
+              ((300, 1200), (5, 5), (1, 1)), ((133, 776), (4, 4), (1, 1)), ((200, 2100), (4, 4), (2, 2)),
+              ((70, 880), (5, 5), (2, 2)), ((31, 224), (4, 4), (1, 1)), ((45, 8), (5, 5), (1, 1)),
+              ((1000, 4100), (5, 5), (1, 1)), ((1200, 1764), (5, 5), (2, 2)), ((5, 444), (5, 5), (2, 2)),
+              ((9, 8), (4, 4), (2, 2))]
 
 
 @pytest.mark.parametrize("shape,window,stride", POOL_CASES)
@@ -784,6 +791,26 @@ def test_pool_bit_exact(dev, shape, window, stride):
         assert np.array_equal(got[:ref.size].reshape(ref.shape), ref)
         assert np.all(got[ref.size:] == -7.0)
         dx.free(); dout.free()
+
+
+@pytest.mark.parametrize("window,stride", [((2, 2), (2, 2)), ((3, 3), (1, 1)), ((5, 5), (2, 2)), ((4, 4), (1, 1)),
+                                           ((3, 2), (1, 3))])
+def test_pool_signed_zeros_and_nans_follow_the_reference_order(dev, window, stride):
+    """The reference keeps the first of equal maxima (strictly greater replaces) and
+    skips NaNs; which of +0 and -0 a window returns shows whether a kernel visits the
+    taps in the reference's order.  Compared bit for bit."""
+    _say("pool zeros/nans", window, stride)
+    rng = np.random.default_rng(1050 + window[0] * 10 + stride[0])
+    shape = (150, 1320)
+    x = rng.choice(np.array([0.0, -0.0, -1.0, np.nan, -2e6], dtype=np.float32), size=shape,
+                   p=[0.3, 0.3, 0.2, 0.1, 0.1]).astype(np.float32)
+    ref = o.fpool(x, window, stride)
+    dx, dout = dev.array(x), dev.empty(ref.size)
+    dev.fpool(dx, dout, shape[0], shape[1], window, stride)
+    got = dout.download().reshape(ref.shape)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    assert np.signbit(ref).any() and (~np.signbit(ref)).any()   # both zeros do occur
+    dx.free(); dout.free()
 
 
 # ---- extended (fused) builtins ----------------------------------------------------

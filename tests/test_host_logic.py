@@ -46,6 +46,22 @@ def test_pool_plan_stays_off_the_staged_kernel_when_the_stride_overflows_32_bits
     assert capi.fpool_plan(64, 100000, (5, 5), (2, 5))[0] == 0      # of 1436 floats: only four do
 
 
+def test_pool_plan_marches_over_square_windows_of_four_and_five():
+    """Kernel 3 takes overlapping square windows of 4 and 5 at stride 1 or 2 when the
+    image rows start on 16 bytes; everything else stays where it was."""
+    for window, stride in (((4, 4), (1, 1)), ((4, 4), (2, 2)), ((5, 5), (1, 1)), ((5, 5), (2, 2))):
+        kernel, band, lds = capi.fpool_plan(8192, 8192, window, stride)
+        assert kernel == 3 and lds == 0 and 8 <= band <= 8192, (window, stride, kernel, band, lds)
+        assert capi.fpool_plan(8192, 8190, window, stride)[0] == 2            # rows off 16 bytes
+        assert capi.fpool_plan(8192, 8192, window, stride, input_aligned=False)[0] == 2
+    assert capi.fpool_plan(8192, 8192, (4, 4), (4, 4))[0] == 1
+    assert capi.fpool_plan(8192, 8192, (5, 5), (3, 3))[0] == 2
+    assert capi.fpool_plan(8192, 8192, (5, 4), (1, 1))[0] == 2
+    assert capi.fpool_plan(8192, 8192, (3, 3), (1, 1))[0] == 2
+    # short images: one band of all the output rows
+    assert capi.fpool_plan(9, 8, (5, 5), (1, 1))[:2] == (3, 5)
+
+
 def test_probe_library_exports_what_the_benchmark_calls():
     import bench
     lib = C.CDLL(bench.LIB_PROBES)
