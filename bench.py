@@ -53,7 +53,7 @@ TRAFFIC_KERNELS = {  # operation -> name fragments of the kernels one call launc
     "fcopy": ["<CopyOp,"], "ffill": ["<FillOp,"], "flogloss": ["<LogLossOp,"], "fmulconcat": ["<ScaleOp,"],
     "frelu": ["<ReluOp,"], "fsoftmax": ["expSumKernel", "finishSumKernel", "<SoftmaxScaleOp,"],
     "ftranspose": ["transpose"], "fmatmul": ["matmulKernel<"], "fconv2d": ["conv2d"], "fpool": ["poolSquareKernel"],
-    "fpool_3x3_stride2": ["poolStagedKernel"],
+    "fpool_3x3_stride2": ["poolStagedKernel<3,3"], "fpool_5x5_stride2": ["poolMarchKernel<5,2"],
 }
 
 
@@ -333,6 +333,16 @@ def summarise_into_roofline(result):
                                 "buffers_rotated": True}
         parts.append(f"ragged matmuls {min(v['frac_hbm_peak'] for v in entries.values()):.3f}-"
                      f"{max(v['frac_hbm_peak'] for v in entries.values()):.3f} of HBM peak on compulsory bytes")
+    mid = result.get("matmul_mid_size")
+    if mid:
+        entries = {k: v for k, v in mid.items() if k.startswith("fmatmul")}
+        mlp = {k: v for k, v in entries.items() if v["M"] * v["N"] * v["K"] == 1024 * 4096 * 1024}
+        roof["matmul_mid_size"] = {k: {"frac_mfma": v["frac_mfma_fp32_peak"], "cold_frac_mfma": v["cold_frac_mfma_fp32_peak"],
+                                       "us": v["us"]} for k, v in entries.items()}
+        parts.append(f"MLP-shape matmuls {min(v['frac_mfma_fp32_peak'] for v in mlp.values()):.3f}-"
+                     f"{max(v['frac_mfma_fp32_peak'] for v in mlp.values()):.3f} of fp32 MFMA peak settled "
+                     f"({min(v['cold_frac_mfma_fp32_peak'] for v in mlp.values()):.3f}-"
+                     f"{max(v['cold_frac_mfma_fp32_peak'] for v in mlp.values()):.3f} cold)")
     return "summary: " + "; ".join(parts)
 
 
@@ -469,6 +479,19 @@ def bench_next_builtins(dev, dx, n, args):
     report("fpool_3x3_stride2", f"{h}x{w} image, max, window 3x3, stride 2x2", ms, 4 * (h * w + oh3 * ow3))
     for t in dpool3:
         t.free()
+    # a stride-1 window (as much written as read) and a 5x5 one (the marching kernel)
+    for key, win, stride in (("fpool_3x3_stride1", 3, 1), ("fpool_5x5_stride2", 5, 2)):
+        oh, ow = (h - win) // stride + 1, (w - win) // stride + 1
+        dp = [dev.empty(oh * ow) for _ in range(R)]
+        ms = time_kernel(dev, lambda i: dev.fpool(dimgs[i % R], dp[i % R], h, w, (win, win), (stride, stride)),
+                         args.warmup, args.steps)
+        report(key, f"{h}x{w} image, max, window {win}x{win}, stride {stride}x{stride}", ms, 4 * (h * w + oh * ow))
+        got = dp[0].download((oh, ow))[:4, :64]
+        want = np.lib.stride_tricks.sliding_window_view(img[:(4 - 1) * stride + win, :(64 - 1) * stride + win],
+                                                        (win, win))[::stride, ::stride].max(axis=(2, 3))
+        assert np.array_equal(got, want), f"{key} output is wrong"
+        for t in dp:
+            t.free()
     got = dpools[0].download((h // 2, w // 2))[:8]
     assert np.array_equal(got, img[:16].reshape(8, 2, w // 2, 2).max(axis=(1, 3))), "pool output is wrong"
     for t in dimgs + dpools + [dk]:
@@ -679,13 +702,24 @@ def bench_ragged(dev, args):
     return out
 
 
+MID_SETTLE_S = 0.03   # matrix work before the settled timing: what the clock takes to settle
+MID_BATCH = 20        # calls between the two events of one settled sample
+
+
 def bench_matmul_mid(dev, args):
     """Matmuls between the two extremes: the MLP configuration's products (batch 1024,
-    1024 -> 4096 -> 1024, forward and gradient graphs) and a few cubes.  Too short for the
-    clock to settle, so they are timed as a graph meets them: a handful of untimed calls,
-    then calls issued back to back over four sets of operands, events around each call
-    (a split contraction's reduction kernel included)."""
-    out = {"timing": "per call, issued back to back over 4 sets of operands, events around each call"}
+    1024 -> 4096 -> 1024, forward and gradient graphs) and a few cubes.  Two figures
+    per shape, over four rotating sets of operands (a split contraction's reduction
+    kernel included in both):
+      us        the time per call inside a running job: 30 ms of the same calls first
+                (the clock has settled, as for the 4096^3 figure), then the mean of
+                20 calls issued back to back between two events, median of 5 such runs;
+      cold_us   as a graph evaluated on an idle device meets it: after a synchronize and
+                50 ms of sleep, six untimed calls, then the median of calls each between
+                its own pair of events (the event records add about 2 us per call)."""
+    out = {"timing": f"us: after {MID_SETTLE_S * 1e3:.0f} ms of the same calls, mean of {MID_BATCH} calls back to back "
+                     "between two events, median of 5 runs; cold_us: after 50 ms idle, 6 untimed calls, median of "
+                     "calls each between its own events; 4 rotating sets of operands"}
     rng = np.random.default_rng(12)
     reps = max(20, args.steps)
     sets = 4
@@ -697,16 +731,35 @@ def bench_matmul_mid(dev, args):
         dbs = device_copies(dev, dev.array(rng.standard_normal(sb, dtype=np.float32)), k * n, sets)
         dcs = [dev.empty(m * n) for _ in range(sets)]
         call = lambda i: dev.fmatmul(ta, tb, das[i % sets], dbs[i % sets], dcs[i % sets], m, n, k)
-        t = float(np.median(time_calls(dev, call, 6, reps))) * 1e-3
-        config, splits, tile = dev.fmatmul_plan(m, n, k)
         flops = 2.0 * m * n * k
+        # cold first (the device has just been idle: uploads and allocation)
+        dev.synchronize()
+        time.sleep(0.05)
+        cold = float(np.median(time_calls(dev, call, 6, reps))) * 1e-3
+        # settled: enough of the same calls to fill MID_SETTLE_S at the cold rate, then batches
+        for i in range(int(MID_SETTLE_S / cold) + 1):
+            call(i)
+        samples = []
+        for _ in range(5):
+            first = dev.record()
+            for i in range(MID_BATCH):
+                call(i)
+            last = dev.record()
+            dev.synchronize()
+            samples.append(first.elapsed_ms(last) * 1e-3 / MID_BATCH)
+            first.release()
+            last.release()
+        t = float(np.median(samples))
+        config, splits, tile = dev.fmatmul_plan(m, n, k)
         name = f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'} {m}x{n}x{k}"
         out[name] = {"M": m, "N": n, "K": k, "us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1),
                      "frac_mfma_fp32_peak": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
+                     "cold_us": round(cold * 1e6, 1),
+                     "cold_frac_mfma_fp32_peak": round(flops / cold / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
                      "tile": "x".join(map(str, tile)), "k_splits": splits}
         log(f"{name:34s} {t * 1e6:8.1f} us  {flops / t / 1e12:6.1f} TFLOP/s  "
-            f"({flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS * 100:.0f} % of the fp32 matrix peak; "
-            f"tile {'x'.join(map(str, tile))}, {splits} k-split(s))")
+            f"({flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS * 100:.0f} % of the fp32 matrix peak; cold {cold * 1e6:.1f} us, "
+            f"{flops / cold / 1e12 / MFMA_FP32_PEAK_TFLOPS * 100:.0f} %; tile {'x'.join(map(str, tile))}, {splits} k-split(s))")
         for x in das + dbs + dcs:
             x.free()
     return out

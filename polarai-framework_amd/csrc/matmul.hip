@@ -465,7 +465,9 @@ struct TileConfig {
   int bm, bn, bk;
   int residentGroups; // groups of this shape one CU holds (LDS, lanes)
   // Microseconds per k-step, measured with every CU busy (cold clock, as a lone
-  // launch in a graph finds it): stepAlone with one group on the CU, and what
+  // launch in a graph finds it; a settled clock runs them 7-10 % faster, the
+  // 128x128 tile with one group per CU 22 %, for which its entry sits between
+  // the two): stepAlone with one group on the CU, and what
   // every co-resident group adds once the groups no longer hide in each other's
   // latency; a step with r groups resident takes max(stepAlone, r * stepPerGroup).
   float stepAlone, stepPerGroup;
@@ -473,7 +475,7 @@ struct TileConfig {
 // order = the switch in matmulWithEpilogue
 constexpr TileConfig kConfigs[] = {
     {256, 256, 32, 1, 8.2f, 8.2f},   // 4x4 waves of 64x64: one group per CU; 7.8 warm, 8.4-9.0 cold
-    {128, 128, 32, 2, 2.6f, 2.28f},  // 2x4 waves of 64x32, tiles fetched two steps ahead
+    {128, 128, 32, 2, 2.4f, 2.28f},  // 2x4 waves of 64x32, tiles fetched two steps ahead (alone: 2.6 cold, 2.04 settled)
     {64, 64, 32, 4, 0.79f, 0.74f},   // 2x2 waves of 32x32, two steps ahead
     {128, 32, 32, 3, 0.85f, 0.77f},  // skinny N
     {32, 128, 32, 3, 0.85f, 0.77f},  // skinny M

@@ -141,5 +141,21 @@ def test_conv2d_pool_full_size(dev):
     got = dout.download((h // 2, w // 2))
     assert np.array_equal(got, o.fpool(x, (2, 2), (2, 2)))
     assert np.array_equal(got, x.reshape(h // 2, 2, w // 2, 2).max(axis=(1, 3)))
-    for t in (dx, dk, dout):
+    dout.free()
+    # overlapping windows: the staged kernel (3x3) and the marching kernel (5x5), against the oracle and
+    # against a size-independent property: pooling with window a then window b at stride 1 is pooling
+    # with window a + b - 1 (max is associative), so 3x3 of 3x3 equals 5x5
+    for window, stride in (((3, 3), (1, 1)), ((5, 5), (2, 2)), ((5, 5), (1, 1))):
+        print("fpool", window, stride, flush=True)
+        oh, ow = (h - window[0]) // stride[0] + 1, (w - window[1]) // stride[1] + 1
+        dout = dev.empty(oh * ow)
+        dev.fpool(dx, dout, h, w, window, stride)
+        assert np.array_equal(dout.download((oh, ow)), o.fpool(x, window, stride))
+        dout.free()
+    d3, d33, d5 = dev.empty((h - 2) * (w - 2)), dev.empty((h - 4) * (w - 4)), dev.empty((h - 4) * (w - 4))
+    dev.fpool(dx, d3, h, w, (3, 3), (1, 1))
+    dev.fpool(d3, d33, h - 2, w - 2, (3, 3), (1, 1))
+    dev.fpool(dx, d5, h, w, (5, 5), (1, 1))
+    assert np.array_equal(d33.download(), d5.download())
+    for t in (dx, dk, d3, d33, d5):
         t.free()
