@@ -53,7 +53,8 @@ TRAFFIC_KERNELS = {  # operation -> name fragments of the kernels one call launc
     "fcopy": ["<CopyOp,"], "ffill": ["<FillOp,"], "flogloss": ["<LogLossOp,"], "fmulconcat": ["<ScaleOp,"],
     "frelu": ["<ReluOp,"], "fsoftmax": ["expSumKernel", "finishSumKernel", "<SoftmaxScaleOp,"],
     "ftranspose": ["transpose"], "fmatmul": ["matmulKernel<"], "fconv2d": ["conv2d"], "fpool": ["poolSquareKernel"],
-    "fpool_3x3_stride2": ["poolStagedKernel<3,3"], "fpool_5x5_stride2": ["poolMarchKernel<5,2"],
+    "fpool_3x3_stride2": ["poolStagedKernel<3,3,true> stride 2"], "fpool_3x3_stride1": ["poolStagedKernel<3,3,true> stride 1"],
+    "fpool_5x5_stride2": ["poolMarchKernel<5,2"],
 }
 
 
