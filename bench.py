@@ -384,6 +384,26 @@ def time_calls(dev, fn, warmup, reps):
     return ms
 
 
+def time_batches(dev, fn, warmup, batch, runs=5):
+    """Seconds per call of `batch` calls issued back to back between ONE pair of
+    events (median of `runs` such batches): what a stream of these calls takes per
+    call.  An event between every two calls, as time_calls records, puts a marker
+    packet between the kernels and costs each call about 3 us."""
+    for i in range(warmup):
+        fn(i)
+    samples = []
+    for r in range(runs):
+        first = dev.record()
+        for i in range(batch):
+            fn(warmup + r * batch + i)
+        last = dev.record()
+        dev.synchronize()
+        samples.append(first.elapsed_ms(last) * 1e-3 / batch)
+        first.release()
+        last.release()
+    return float(np.median(samples))
+
+
 def device_copies(dev, src, count, copies):
     """`copies` buffers holding the same `count` floats as `src` (src is the first)."""
     out = [src]
@@ -454,8 +474,8 @@ def bench_next_builtins(dev, dx, n, args):
     dxs = device_copies(dev, dx, n, R)
     ms = time_kernel(dev, lambda i: dev.frelu(dxs[i % R], douts[i % R]), args.warmup, args.steps)
     report("frelu", f"{n} elements, 1R+1W", ms, 8 * n)
-    # fsoftmax is three launches (partial sums, total, scale): events around each call
-    ms = time_calls(dev, lambda i: dev.fsoftmax(dxs[i % R], douts[i % R]), args.warmup, args.steps)
+    # fsoftmax is three launches (partial sums, total, scale): time per call of a stream of calls
+    ms = [time_batches(dev, lambda i: dev.fsoftmax(dxs[i % R], douts[i % R]), args.warmup, max(8, args.steps // 2)) * 1e3]
     report("fsoftmax", f"{n} elements over the whole tensor, 2R+1W (sum pass, scale pass)", ms, 12 * n)
     for t in douts + dxs[1:]:
         t.free()
@@ -657,9 +677,11 @@ def bench_ragged(dev, args):
     """The ragged configuration: fadd/fmul on 1 000 003 elements and the two matmul
     shapes 65536x127x33 / 33x65536x127 under both readings of the triple, (M, K, N)
     and (M, N, K).  These are small: both roofline bounds are reported.  `us` is
-    the time per call of calls issued back to back (events around each call, so
-    kernels that follow a first one are included); `first_kernel_us` is the
-    execution time of the call's first kernel alone.  Every kernel cycles through
+    the time per call of a stream of calls (batches of 20 between one pair of
+    events, median of 5; kernels that follow a first one are included),
+    `us_event_per_call` the same with an event recorded between every two calls
+    (about 3 us more: the marker packets), `first_kernel_us` the execution time
+    of the call's first kernel alone.  Every kernel cycles through
     as many sets of operands as it takes to exceed the Infinity Cache, so no call
     finds its operands where the previous call left them."""
     out = {"buffers_rotated": True, "rotated_bytes": RAGGED_ROTATE_BYTES}
@@ -687,16 +709,18 @@ def bench_ragged(dev, args):
         dbs = device_copies(dev, dev.array(rng.standard_normal((k, nn), dtype=np.float32)), k * nn, sets)
         dcs = [dev.empty(m * nn) for _ in range(sets)]
         call = lambda i: dev.fmatmul(0, 0, das[i % sets], dbs[i % sets], dcs[i % sets], m, nn, k)
-        t = float(np.mean(time_calls(dev, call, max(3, args.warmup, sets), reps))) * 1e-3
+        with_events = float(np.mean(time_calls(dev, call, max(3, args.warmup, sets), reps))) * 1e-3
+        t = time_batches(dev, call, sets, 20)
         first = float(np.mean(time_kernel(dev, call, sets, reps))) * 1e-3
         out[f"fmatmul_f_f {label}"] = {"M": m, "N": nn, "K": k, "us": round(t * 1e6, 2),
+                                       "us_event_per_call": round(with_events * 1e6, 2),
                                        "first_kernel_us": round(first * 1e6, 2),
                                        "GFLOP/s": round(flops / t / 1e9, 1),
                                        "frac_mfma_fp32_peak": round(flops / t / 1e12 / MFMA_FP32_PEAK_TFLOPS, 4),
                                        "min_bytes_GB/s": round(nbytes / t / 1e9, 1),
                                        "frac_hbm_peak": round(nbytes / t / 1e9 / HBM_PEAK_GBS, 4),
                                        "buffer_sets": sets}
-        log(f"fmatmul {label}: {t * 1e6:7.1f} us per call (first kernel {first * 1e6:.1f} us)  "
+        log(f"fmatmul {label}: {t * 1e6:7.1f} us per call ({with_events * 1e6:.1f} with an event per call; first kernel {first * 1e6:.1f} us)  "
             f"{flops / t / 1e12:6.2f} TFLOP/s  {nbytes / t / 1e9:7.1f} GB/s of compulsory traffic  ({sets} operand sets)")
         for x in das + dbs + dcs:
             x.free()
@@ -740,17 +764,7 @@ def bench_matmul_mid(dev, args):
         # settled: enough of the same calls to fill MID_SETTLE_S at the cold rate, then batches
         for i in range(int(MID_SETTLE_S / cold) + 1):
             call(i)
-        samples = []
-        for _ in range(5):
-            first = dev.record()
-            for i in range(MID_BATCH):
-                call(i)
-            last = dev.record()
-            dev.synchronize()
-            samples.append(first.elapsed_ms(last) * 1e-3 / MID_BATCH)
-            first.release()
-            last.release()
-        t = float(np.median(samples))
+        t = time_batches(dev, call, 0, MID_BATCH)
         config, splits, tile = dev.fmatmul_plan(m, n, k)
         name = f"fmatmul_{'t' if ta else 'f'}_{'t' if tb else 'f'} {m}x{n}x{k}"
         out[name] = {"M": m, "N": n, "K": k, "us": round(t * 1e6, 1), "TFLOP/s": round(flops / t / 1e12, 1),
