@@ -202,8 +202,12 @@ int polar_hip_fmatmul(polar_hip_device* dev, int transA, int transB,
 /* How polar_hip_fmatmul would compute an M x N x K product (no counterpart in
  * the reference; for tuning and tests): the tile configuration its planner
  * picks (an index into the library's table; -1 for the shapes taken by the
- * short-contraction kernels), the number of parts the contraction is split
- * into, and, if tile is not null, the tile's extent along M, N and K. */
+ * short-contraction and long-contraction kernels), the number of parts the
+ * contraction is split into, and, if tile is not null, the tile's extent along
+ * M, N and K.  The parts' partial products are added in split order, by a
+ * second kernel or (up to eight parts, where that is estimated to be cheaper)
+ * by the work-group that finishes a tile last: same bits on every run either
+ * way. */
 int polar_hip_fmatmul_plan(polar_hip_device* dev, uint64_t m, uint64_t n,
                            uint64_t k, int* tile_config, uint32_t* splits,
                            uint32_t tile[3]);

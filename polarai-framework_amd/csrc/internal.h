@@ -88,6 +88,11 @@ struct polar_hip_device {
   std::mutex workspaceMu;
   void* workspace = nullptr;
   uint64_t workspaceBytes = 0;
+  // One arrival counter per C tile of a split contraction whose last-arriving
+  // work-group adds the partial products itself (matmul.hip).  Allocated and
+  // zeroed when the device is opened; the group that completes a tile sets its
+  // counter back to zero, so every launch finds zeros.  Used under workspaceMu.
+  uint32_t* tileCounters = nullptr;
   // Transfers queued directly out of or into blocks of polar_hip_host_alloc are
   // numbered per device handle; directDone is the highest number known to be
   // complete, learnt from whatever the caller waits for anyway (an event
@@ -127,6 +132,7 @@ constexpr uint64_t kWorkspaceBytes = 256ull << 20;
 // contents undefined), grown if it was smaller.  Caller holds dev->workspaceMu.
 // Fails for a request above kWorkspaceBytes.
 int workspaceFor(polar_hip_device* dev, uint64_t bytes, void** area); // runtime.hip
+constexpr uint32_t kTileCounters = 16384;  // entries of polar_hip_device::tileCounters
 
 // Every kernel of the library is launched through here.  Normally a plain
 // launch on the device's stream; when a timing pair is armed, the launch

@@ -66,6 +66,10 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 // then fall on 32 different banks (with BX + 4 they fell on 8).
 template <int BX, bool KCONTIG> constexpr int ldsPitch() { return BX + (KCONTIG ? 1 : 4); }
 constexpr int kXcds = 8;
+#ifndef FUSED_SPLITS
+#define FUSED_SPLITS 8
+#endif
+constexpr uint32_t kFusedSplits = FUSED_SPLITS;  // most parts of K that are added by the last group of a tile
 
 struct MatmulArgs {
   const float* A;
@@ -81,6 +85,14 @@ struct MatmulArgs {
   int epilogue;
   const float* bias;  // M x N, dense (the framework's fadd does not broadcast)
   float scaleAcc, scaleBias;
+  // Split contraction whose last-arriving work-group adds the partial products
+  // itself: one arrival counter per C tile (all zero when the kernel starts)
+  // and the final output.  C then points at the workspace, where split s of
+  // tile t keeps its BM x BN accumulators at [(t kSplits + s) BM BN], in the
+  // order the lanes hold them.  Null: partial products go to C as whole
+  // matrices, one per split, for a second kernel to add.
+  uint32_t* tileCounters;
+  float* finalC;
 };
 
 // Fetch of one operand tile (BX x BK) from HBM into registers, and its store
@@ -322,6 +334,71 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
     }
   }
 
+  float* finalOut = out;
+  bool finalValues = p.kSplits == 1;  // what is stored is an element of the product (the epilogue applies)
+  if (p.tileCounters != nullptr) {  // (uniform)
+    // Partial products meet in the workspace, and the group that arrives last
+    // at a tile adds them.  The XCDs' L2 caches are not coherent with each
+    // other, and a device-scope fence per group (write back and invalidate the
+    // whole L2) costs more than the product: 1024x1024x4096 in four parts 168
+    // us with fences against 82 with a second kernel.  So the partial products
+    // leave through write-through stores (16 bytes per lane, the lanes of a
+    // store side by side: whole lines, which matters for stores that go to
+    // memory as they are) and are ordered by hand: every thread
+    // waits until its stores are acknowledged, the group meets at a barrier,
+    // and only then one thread counts the group in.  The group that sees
+    // kSplits - 1 earlier arrivals is the last; what the others stored was in
+    // memory before they counted themselves in.  Its loads of their partial
+    // products are ordinary ones: a launch starts with every L2 invalidated, and
+    // until now nothing in this launch has read those lines, so they cannot be
+    // stale in this XCD's L2.  It adds the partial products in split order --
+    // its own from registers, in its place -- so the sum does not depend on
+    // which group came last, and leaves the counter at zero for the next
+    // launch.
+    __shared__ uint32_t arrivedBefore;
+    const uint32_t tile = blockIdx.x % tiles;
+    constexpr uint32_t kTileFloats = uint32_t(BM) * BN;
+    float* const partials = p.C + size_t(tile) * p.kSplits * kTileFloats;
+    float* const mine = partials + size_t(split) * kTileFloats;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; r += 4)
+          streamStore(v4f{acc[i][j][r], acc[i][j][r + 1], acc[i][j][r + 2], acc[i][j][r + 3]},
+                      reinterpret_cast<v4f*>(mine + (((i * TN + j) * 4 + r / 4) * NT + t) * 4));
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (t == 0)
+      arrivedBefore = __hip_atomic_fetch_add(&p.tileCounters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (arrivedBefore != p.kSplits - 1) return;
+    if (t == 0) __hip_atomic_store(&p.tileCounters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        // quarter q of the block's sixteen values: [((block 4 + q) lanes + lane) 4]
+        auto partOf = [&](uint32_t s) {
+          const float* const from = partials + size_t(s) * kTileFloats + (((i * TN + j) * 4) * NT + t) * 4;
+          v16f v;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const v4f piece = *reinterpret_cast<const v4f*>(from + q * NT * 4);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) v[4 * q + c] = piece[c];
+          }
+          return v;
+        };
+        v16f total = split == 0 ? acc[i][j] : partOf(0);
+        for (uint32_t s = 1; s < p.kSplits; ++s) total += s == split ? acc[i][j] : partOf(s);
+        acc[i][j] = total;
+      }
+    finalOut = p.finalC;
+    finalValues = true;
+  }
+
   // Accumulator block layout of the 32x32 MFMA: register r of lane l holds
   // row 8*(r/4) + 4*(l/32) + r%4, column l%32.
 #pragma unroll
@@ -335,9 +412,9 @@ __global__ __launch_bounds__(WM* WN * 64) void matmulKernel(MatmulArgs p) {
             m0 + wm * WTM + i * 32 + 8 * (r / 4) + 4 * (lane / 32) + (r % 4);
         if (!EDGE || (row < p.M && col < p.N)) {
           const size_t idx = size_t(row) * p.N + col;
-          out[idx] = p.kSplits > 1 ? acc[i][j][r]
-                                   : applyEpilogue(p.epilogue, acc[i][j][r], p.bias,
-                                                   p.scaleAcc, p.scaleBias, idx);
+          finalOut[idx] = finalValues ? applyEpilogue(p.epilogue, acc[i][j][r], p.bias,
+                                                      p.scaleAcc, p.scaleBias, idx)
+                                      : acc[i][j][r];
         }
       }
     }
@@ -415,7 +492,7 @@ int launchLayout(polar_hip_device* dev, const MatmulArgs& p, bool vec, bool edge
 
 template <int BM, int BN, int BK, int WM, int WN, int PF = 1>
 int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
-               uint32_t splits) {
+               uint32_t splits, bool lastGroupAdds) {
   MatmulArgs p = p0;
   p.tilesM = (p.M + BM - 1) / BM;
   p.tilesN = (p.N + BN - 1) / BN;
@@ -442,18 +519,28 @@ int launchTile(polar_hip_device* dev, bool ta, bool tb, const MatmulArgs& p0,
   // call's two kernels
   std::unique_lock<std::mutex> workspaceLock(dev->workspaceMu, std::defer_lock);
   void* workspace = nullptr;
+  // Up to kFusedSplits parts of K: the group that arrives last at a tile adds
+  // the tile's partial products itself (they sit in the workspace tile by tile)
+  // and no second kernel runs.  With more parts one group would add for too
+  // long while the rest of the chip idles; those keep the reduction kernel.
+  const uint64_t tiles = uint64_t(p.tilesM) * p.tilesN;
+  const uint64_t fusedBytes = tiles * splits * BM * BN * sizeof(float);
+  const bool fused = lastGroupAdds && splits > 1 && splits <= kFusedSplits && tiles <= kTileCounters && fusedBytes <= kWorkspaceBytes;
+  p.tileCounters = nullptr;
+  p.finalC = c;
   if (splits > 1) {
     workspaceLock.lock();
-    int st = workspaceFor(dev, count * splits * sizeof(float), &workspace);
+    int st = workspaceFor(dev, fused ? fusedBytes : count * splits * sizeof(float), &workspace);
     if (st != POLAR_HIP_OK) return st;
     p.C = static_cast<float*>(workspace);
+    if (fused) p.tileCounters = dev->tileCounters;
   }
   int st;
   if (!ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, PF, false, false>(dev, p, vec, edge);
   else if (!ta && tb) st = launchLayout<BM, BN, BK, WM, WN, PF, false, true>(dev, p, vec, edge);
   else if (ta && !tb) st = launchLayout<BM, BN, BK, WM, WN, PF, true, false>(dev, p, vec, edge);
   else st = launchLayout<BM, BN, BK, WM, WN, PF, true, true>(dev, p, vec, edge);
-  if (splits > 1 && st == POLAR_HIP_OK) {
+  if (splits > 1 && !fused && st == POLAR_HIP_OK) {
     hipError_t e = launchReduce(dev, static_cast<const float*>(workspace), c, count, splits, p);
     if (e != hipSuccess) st = failHip(e, "splitKReduceKernel");
   }
@@ -489,7 +576,24 @@ constexpr TileConfig kConfigs[] = {
 struct MatmulPlan {
   int config;
   uint32_t splits;
+  bool fused;  // splits > 1: the last group of a tile adds the partial products (no second kernel)
 };
+
+// What adding the partial products of a split contraction costs, in
+// microseconds, either way.  Second kernel: a launch, and every partial
+// product written and read once more.  Last group of a tile: its chain of
+// store acknowledgement, counter and loads (about as long as a launch), the
+// write-through stores of all partial products, and one group reading the
+// other s - 1 partial products of a tile at about 40 GB/s.  (Measured against
+// each other on a settled clock: 3072^3 in four parts 494 -> 454 us, 1024 x
+// 2048 x 4096 160 -> 140, 768^3 19.4 -> 15.7; but 512^3 9.1 -> 10.6 and 300 x
+// 300 x 3000 16.2 -> 20.1, which therefore keep the second kernel.)
+constexpr uint32_t kFusedTileLimit = kTileCounters;
+inline double reduceKernelUs(double m, double n, uint32_t s) { return 4.0 + m * n * 4.0 * (s + 1) / 3.0e6; }
+inline double lastGroupAddsUs(double m, double n, uint32_t s, int bm, int bn) {
+  return 4.0 + m * n * 4.0 * s / 4.0e6 + (s - 1) * double(bm) * bn * 4.0 / 40.0e3;
+}
+inline bool lastGroupMayAdd(uint32_t s, double tiles) { return s > 1 && s <= kFusedSplits && tiles <= kFusedTileLimit; }
 
 // Estimated microseconds of every tile shape and split count; the cheapest
 // wins.  The groups run in rounds of (CUs x resident groups); a k-step of a
@@ -504,9 +608,11 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
   constexpr int kCount = int(sizeof(kConfigs) / sizeof(kConfigs[0]));
   double usOf[kCount], tilesOf[kCount];
   uint32_t splitsOf[kCount];
+  bool fusedOf[kCount];
   for (int c = 0; c < kCount; ++c) {
     usOf[c] = 1e30;
     splitsOf[c] = 1;
+    fusedOf[c] = false;
     const TileConfig& t = kConfigs[c];
     const double tiles = double((m + t.bm - 1) / t.bm) * ((n + t.bn - 1) / t.bn);
     const uint32_t kSteps = (k + t.bk - 1) / t.bk;
@@ -523,10 +629,16 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
       double perStep = fullRounds * stepUs(t.residentGroups);
       if (rest > 0.5) perStep += stepUs(std::ceil(rest / computeUnits - 1e-9));
       double us = ((kSteps + s - 1) / s) * perStep + 4.0 + 2.5 * t.stepAlone;
-      if (s > 1) us += 4.0 + double(m) * n * 4.0 * (s + 1) / 3.0e6;
+      bool fused = false;
+      if (s > 1) {
+        const double second = reduceKernelUs(m, n, s), last = lastGroupAddsUs(m, n, s, t.bm, t.bn);
+        fused = lastGroupMayAdd(s, tiles) && last < second;
+        us += fused ? last : second;
+      }
       if (us < usOf[c]) {
         usOf[c] = us;
         splitsOf[c] = s;
+        fusedOf[c] = fused;
       }
     }
     tilesOf[c] = tiles;
@@ -543,7 +655,7 @@ MatmulPlan planMatmul(uint32_t m, uint32_t n, uint32_t k, int computeUnits) {
   int best = cheapest;
   for (int c = 0; c < kCount; ++c)
     if (splitsOf[c] == splitsOf[cheapest] && usOf[c] <= usOf[cheapest] * 1.04 && tilesOf[c] < tilesOf[best]) best = c;
-  return MatmulPlan{best, splitsOf[best]};
+  return MatmulPlan{best, splitsOf[best], fusedOf[best]};
 }
 
 } // namespace
@@ -558,7 +670,7 @@ static_assert(kConfigCount == POLAR_HIP_MATMUL_TILE_CONFIGS, "the header states 
 int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const float* a,
                        const float* b, float* c, uint64_t m, uint64_t n, uint64_t k,
                        int epilogue, const float* bias, float scaleAcc, float scaleBias,
-                       MatmulPlan forced = MatmulPlan{-1, 1}) {
+                       MatmulPlan forced = MatmulPlan{-1, 1, false}) {
   POLAR_HIP_REQUIRE(dev != nullptr, "dev is null");
   if (m == 0 || n == 0) return POLAR_HIP_OK;
   POLAR_HIP_REQUIRE(c != nullptr, "null output");
@@ -569,7 +681,7 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   POLAR_HIP_REQUIRE(epilogue != kEpiAddSigmoid || bias != nullptr, "null bias");
   POLAR_HIP_TRY(hipSetDevice(dev->ordinal));
   MatmulArgs p{a, b, c, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
-               static_cast<uint32_t>(k), 0, 0, 1, 0, epilogue, bias, scaleAcc, scaleBias};
+               static_cast<uint32_t>(k), 0, 0, 1, 0, epilogue, bias, scaleAcc, scaleBias, nullptr, c};
   if (k == 0) {
     // Empty contraction: the reference's loop leaves acc = 0 and stores it.
     if (epilogue == kEpiNone) return polar_hip_ffill(dev, 0.0f, c, m * n);
@@ -589,16 +701,16 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   const MatmulPlan plan =
       forced.config < 0 ? planMatmul(p.M, p.N, p.K, dev->info.compute_units) : forced;
   switch (plan.config) {
-  case 0: return launchTile<256, 256, 32, 4, 4, 1>(dev, ta, tb, p, plan.splits);
-  case 1: return launchTile<128, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
-  case 2: return launchTile<64, 64, 32, 2, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 3: return launchTile<128, 32, 32, 4, 1, 2>(dev, ta, tb, p, plan.splits);
-  case 4: return launchTile<32, 128, 32, 1, 4, 2>(dev, ta, tb, p, plan.splits);
-  case 5: return launchTile<32, 32, 32, 1, 1, 1>(dev, ta, tb, p, plan.splits);
-  case 6: return launchTile<256, 128, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits);
-  case 7: return launchTile<128, 256, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
-  case 8: return launchTile<128, 64, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits);
-  default: return launchTile<64, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits);
+  case 0: return launchTile<256, 256, 32, 4, 4, 1>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 1: return launchTile<128, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 2: return launchTile<64, 64, 32, 2, 2, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 3: return launchTile<128, 32, 32, 4, 1, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 4: return launchTile<32, 128, 32, 1, 4, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 5: return launchTile<32, 32, 32, 1, 1, 1>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 6: return launchTile<256, 128, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 7: return launchTile<128, 256, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  case 8: return launchTile<128, 64, 32, 4, 2, 2>(dev, ta, tb, p, plan.splits, plan.fused);
+  default: return launchTile<64, 128, 32, 2, 4, 2>(dev, ta, tb, p, plan.splits, plan.fused);
   }
 }
 } // namespace
@@ -644,7 +756,7 @@ extern "C" int polar_hip_fmatmul_with_plan(polar_hip_device* dev, int transA, in
   POLAR_HIP_REQUIRE(splits == 1 || m * n * splits * sizeof(float) <= kWorkspaceBytes,
                     "partial products exceed the workspace");
   return matmulWithEpilogue(dev, transA, transB, a, b, c, m, n, k, kEpiNone, nullptr, 1.0f, 1.0f,
-                            MatmulPlan{tile_config, splits});
+                            MatmulPlan{tile_config, splits, splits > 1 && splits <= kFusedSplits});
 }
 
 extern "C" int polar_hip_fmatmul_fsigmoid(polar_hip_device* dev, int transA, int transB,

@@ -140,7 +140,13 @@ int polar_hip_device_open(int ordinal, polar_hip_device** out) {
   d->info.pci_bus_id = p.pciBusID;
   d->info.hbm_bytes = p.totalGlobalMem;
   st = resolveStaticScratch(d);
+  if (st == POLAR_HIP_OK) {
+    e = hipMalloc(reinterpret_cast<void**>(&d->tileCounters), kTileCounters * sizeof(uint32_t));
+    if (e == hipSuccess) e = hipMemset(d->tileCounters, 0, kTileCounters * sizeof(uint32_t));
+    if (e != hipSuccess) st = failHip(e, "hipMalloc / hipMemset (tile counters)");
+  }
   if (st != POLAR_HIP_OK) {
+    if (d->tileCounters) (void)hipFree(d->tileCounters);
     (void)hipStreamDestroy(d->stream);
     delete d;
     return st;
@@ -171,6 +177,7 @@ int polar_hip_device_close(polar_hip_device* dev) {
     for (void* p : kv.second) (void)hipFree(p);
   for (auto& kv : dev->live) (void)hipFree(kv.first);
   if (dev->workspace) (void)hipFree(dev->workspace);
+  if (dev->tileCounters) (void)hipFree(dev->tileCounters);
   for (auto* e : dev->allEvents) {
     (void)hipEventDestroy(e->ev);
     delete e;

@@ -245,6 +245,47 @@ def test_matmul_every_tile_configuration(dev, ta, tb, config):
         db.free()
 
 
+def test_matmul_split_contraction_is_added_by_the_last_group_repeatably(dev):
+    """Up to eight parts of K are added by whichever work-group finishes a tile
+    last (an arrival counter per tile, set back to zero by that group); more
+    parts go through the second kernel.  The sum is taken in split order either
+    way: repeated calls give the same bits, calls of other shapes in between find
+    the counters at zero, and integer data is exact under every plan."""
+    rng = np.random.default_rng(77)
+    shapes = [(768, 768, 768), (1536, 1536, 1536), (1000, 515, 2100), (384, 384, 4096)]
+    data = {}
+    for (m, n, k) in shapes:
+        a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+        b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        data[(m, n, k)] = (dev.array(a), dev.array(b), o.fmatmul(False, False, a, b))
+    for rnd in range(3):                       # the shapes in turn, three times over
+        for (m, n, k), (da, db, ref) in data.items():
+            _say("split contraction", (m, n, k), "round", rnd)
+            dc = dev.array(np.full(m * n, np.nan, dtype=np.float32))
+            dev.fmatmul(False, False, da, db, dc, m, n, k)
+            assert np.array_equal(dc.download((m, n)), ref)
+            for config, splits in ((1, 2), (1, 8), (2, 5), (8, 3), (1, 12), (2, 16)):   # <= 8: last group; more: second kernel
+                dev.ffill(float("nan"), dc)
+                dev.fmatmul_with_plan(False, False, da, db, dc, m, n, k, config, splits)
+                assert np.array_equal(dc.download((m, n)), ref), ((m, n, k), config, splits, rnd)
+            dc.free()
+    # real-valued data: the same bits every time, whichever group arrives last
+    m, n, k = 1536, 1536, 1536
+    a, b = parity.normal(rng, (m, k)), parity.normal(rng, (k, n))
+    da, db = dev.array(a), dev.array(b)
+    outs = []
+    for i in range(6):
+        dc = dev.empty(m * n)
+        dev.fmatmul_with_plan(False, False, da, db, dc, m, n, k, 1, 3)
+        outs.append(dc.download((m, n)))
+        dc.free()
+    for other in outs[1:]:
+        assert np.array_equal(outs[0].view(np.uint32), other.view(np.uint32))
+    assert parity.frobenius_rel_error(outs[0], o.fmatmul(False, False, a, b)) <= parity.MATMUL_FRO_REL
+    for t in [da, db] + [x for v in data.values() for x in v[:2]]:
+        t.free()
+
+
 def test_matmul_plan_is_reported_and_forced_plans_are_checked(dev):
     config, splits, tile = dev.fmatmul_plan(4096, 4096, 4096)
     assert (config, splits, tile) == (0, 1, (256, 256, 32))
