@@ -269,6 +269,24 @@ def test_matmul_split_contraction_is_added_by_the_last_group_repeatably(dev):
                 dev.fmatmul_with_plan(False, False, da, db, dc, m, n, k, config, splits)
                 assert np.array_equal(dc.download((m, n)), ref), ((m, n, k), config, splits, rnd)
             dc.free()
+    # two operand sets of one shape in turn, back to back with nothing waited for in between: the same plan
+    # and the same places in the workspace, different values -- a partial product read from a stale cache
+    # line would be the other set's
+    m, n, k = 700, 900, 2600
+    pair = []
+    for i in range(2):
+        a = rng.integers(-8, 9, (k, m)).astype(np.float32)
+        b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+        pair.append((dev.array(a), dev.array(b), dev.empty(m * n), o.fmatmul(True, False, a, b)))
+    for config, splits in ((1, 4), (2, 7), (0, 2), (9, 3)):
+        for rep in range(4):
+            for da, db, dc, ref in pair:
+                dev.fmatmul_with_plan(True, False, da, db, dc, m, n, k, config, splits)
+        for da, db, dc, ref in pair:
+            assert np.array_equal(dc.download((m, n)), ref), (config, splits)
+    for st in pair:
+        for t in st[:3]:
+            t.free()
     # real-valued data: the same bits every time, whichever group arrives last
     m, n, k = 1536, 1536, 1536
     a, b = parity.normal(rng, (m, k)), parity.normal(rng, (k, n))
