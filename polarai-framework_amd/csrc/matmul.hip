@@ -563,7 +563,7 @@ struct TileConfig {
 constexpr TileConfig kConfigs[] = {
     {256, 256, 32, 1, 8.2f, 8.2f},   // 4x4 waves of 64x64: one group per CU; 7.8 warm, 8.4-9.0 cold
     {128, 128, 32, 2, 2.4f, 2.28f},  // 2x4 waves of 64x32, tiles fetched two steps ahead (alone: 2.6 cold, 2.04 settled)
-    {64, 64, 32, 4, 0.79f, 0.74f},   // 2x2 waves of 32x32, two steps ahead
+    {64, 64, 32, 4, 0.79f, 0.62f},   // 2x2 waves of 32x32, two steps ahead (per group: 0.74 cold, 0.58 settled)
     {128, 32, 32, 3, 0.85f, 0.77f},  // skinny N
     {32, 128, 32, 3, 0.85f, 0.77f},  // skinny M
     {32, 32, 32, 8, 1.0f, 0.22f},    // one wave (0.78 in a long loop; short loops measured 10 % behind the others)
