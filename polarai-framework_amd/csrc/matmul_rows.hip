@@ -370,6 +370,7 @@ bool rowsMatmulApplies(const MatmulCall& c, int computeUnits) {
   if (c.M < kGroupRows * uint32_t(computeUnits) * 3 / 4) return false;  // most CUs get a group of waves
   const uint32_t blocks = blocksFor(c.N), groups = (c.K + 15) / 16;
   if (blocks * groups > 32) return false;  // B must fit the registers
+  if (blocks > 4 && groups > 4) return false;  // (no kernel is built for those: launchGroups)
   if ((reinterpret_cast<uintptr_t>(c.A) & 15u) != 0) return false;
   const uint32_t words = groups * blocks * 256 + groups * 16 + kWaves * areaWordsFor(c.N, c.K);
   return words * sizeof(float) <= kMaxLds;

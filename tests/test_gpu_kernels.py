@@ -361,7 +361,10 @@ def test_matmul_short_contraction_tall_and_wide(dev, ta, tb, mnk):
 LONG_PANEL_SHAPES = [(65536, 33, 127), (65521, 33, 127), (65553, 127, 33), (33, 65536, 127), (65537, 33, 127),
                      (33, 65541, 127), (65599, 64, 128), (49152, 1, 4), (1, 49153, 5), (70001, 17, 63), (16, 70003, 64),
                      (66000, 128, 64), (128, 66001, 33), (65536, 48, 100), (48, 65538, 16), (65536, 65, 17),
-                     (100000, 5, 97), (65567, 17, 5), (70000, 128, 16), (65536, 100, 65), (65536, 15, 113)]
+                     (100000, 5, 97), (65567, 17, 5), (70000, 128, 16), (65536, 100, 65), (65536, 15, 113),
+                     # five or six column blocks with five or six groups of k: too much of B for the kernel that
+                     # keeps it in registers, which must pass these on
+                     (65536, 70, 90), (50011, 81, 95), (49152, 96, 80), (96, 66000, 80)]
 
 
 @pytest.mark.parametrize("misalign", [0, 1])
