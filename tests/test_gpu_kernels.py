@@ -878,7 +878,11 @@ def test_pool_signed_zeros_and_nans_follow_the_reference_order(dev, window, stri
 # ---- extended (fused) builtins ----------------------------------------------------
 
 FUSED_SHAPES = [(256, 10, 784), (64, 64, 64), (33, 127, 4096), (300, 257, 129), (1024, 1024, 512), (5, 3, 0),
-                (2050, 33, 127), (40, 1500, 30), (784, 10, 256), (12, 300, 100)]
+                (2050, 33, 127), (40, 1500, 30), (784, 10, 256), (12, 300, 100),
+                # the kernels for a short contraction with one long dimension and for a long contraction with a
+                # small result, and a split contraction added by the last group of a tile
+                (65536, 33, 127), (65536, 127, 33), (33, 65536, 127), (70001, 17, 63), (33, 127, 65536),
+                (16, 100, 20000), (50011, 81, 95), (768, 768, 768)]
 
 
 @pytest.mark.parametrize("mnk", FUSED_SHAPES)
