@@ -1,5 +1,6 @@
 """Seeded random shapes for the kernels with index arithmetic (matmul in its four
-layouts, transpose, conv2d, pool): small enough for the oracle, awkward enough to
+layouts -- small shapes, and shapes with one long dimension --, transpose, conv2d,
+pool): small enough for the oracle, awkward enough to
 hit every edge path (sizes around the tile sizes, odd pitches, bases off a line).
 Same bars as the fixed-shape tests: bit-exact for transpose/conv2d/pool, 1e-4
 relative Frobenius for matmul."""
@@ -47,6 +48,36 @@ def test_random_matmul(dev, seed):
     got = dc.download()
     assert np.all(got[m * n:] == -7.0)
     assert parity.frobenius_rel_error(got[:m * n].reshape(m, n), o.fmatmul(ta, tb, a, b)) <= parity.MATMUL_FRO_REL
+    for t in (da, db, dc):
+        t.free()
+
+
+@pytest.mark.parametrize("seed", range(36 * SCALE))
+def test_random_matmul_with_one_long_dimension(dev, seed):
+    """The kernels for a short contraction with a long M or N and for a long
+    contraction with a small result, and whatever the dispatch passes on to the
+    tiled kernel when a shape fits none of them.  Integer data: exact under any
+    order of the additions."""
+    rng = np.random.default_rng(5500 + seed)
+    kind = seed % 3
+    if kind == 0:
+        m, n, k = int(rng.integers(40000, 90000)), _dims(rng, 1, 128)[0], _dims(rng, 1, 140)[0]
+    elif kind == 1:
+        m, n, k = _dims(rng, 1, 128)[0], int(rng.integers(40000, 90000)), _dims(rng, 1, 140)[0]
+    else:
+        m, n, k = _dims(rng, 1, 33)[0], _dims(rng, 1, 128)[0], int(rng.integers(16000, 90000))
+    ta, tb = bool(rng.integers(2)), bool(rng.integers(2))
+    mis_a, mis_b, mis_c = (int(rng.choice([0, 0, 1, 3])) for _ in range(3))
+    _say("random long matmul", seed, (m, n, k), ta, tb, "misalign", (mis_a, mis_b, mis_c), "plan", dev.fmatmul_plan(m, n, k))
+    sa, sb = parity.stored_shapes(ta, tb, m, n, k)
+    a = rng.integers(-4, 5, sa).astype(np.float32)
+    b = rng.integers(-4, 5, sb).astype(np.float32)
+    da, db, dc = dev.array(a, mis_a), dev.array(b, mis_b), dev.empty(m * n + 32, mis_c)
+    dev.ffill(-7.0, dc)
+    dev.fmatmul(ta, tb, da, db, dc, m, n, k)
+    got = dc.download()
+    assert np.all(got[m * n:] == -7.0)
+    assert np.array_equal(got[:m * n].reshape(m, n), o.fmatmul(ta, tb, a, b))
     for t in (da, db, dc):
         t.free()
 
