@@ -698,6 +698,7 @@ int matmulWithEpilogue(polar_hip_device* dev, int transA, int transB, const floa
   if (forced.config < 0 && panelMatmulApplies(call, dev->info.compute_units)) return launchPanelMatmul(dev, call);
   if (forced.config < 0 && smallKMatmulApplies(call)) return launchSmallKMatmul(dev, call);
   if (forced.config < 0 && longKMatmulApplies(call)) return launchLongKMatmul(dev, call);
+  if (forced.config < 0 && skinnyMatmulApplies(call)) return launchSkinnyMatmul(dev, call);
   const MatmulPlan plan =
       forced.config < 0 ? planMatmul(p.M, p.N, p.K, dev->info.compute_units) : forced;
   switch (plan.config) {
@@ -730,7 +731,7 @@ extern "C" int polar_hip_fmatmul_plan(polar_hip_device* dev, uint64_t m, uint64_
   // the short-contraction kernels take any layout of such a shape
   const MatmulCall call{nullptr, nullptr, nullptr, static_cast<uint32_t>(m), static_cast<uint32_t>(n),
                         static_cast<uint32_t>(k), false, false, kEpiNone, nullptr, 1.0f, 1.0f};
-  if (smallKMatmulApplies(call) || longKMatmulApplies(call)) {
+  if (smallKMatmulApplies(call) || longKMatmulApplies(call) || skinnyMatmulApplies(call)) {
     *tile_config = -1;
     *splits = 1;
     if (tile != nullptr) tile[0] = tile[1] = tile[2] = 0;

@@ -66,4 +66,9 @@ int launchRowsMatmul(polar_hip_device* dev, const MatmulCall& call);
 bool longKMatmulApplies(const MatmulCall& call);
 int launchLongKMatmul(polar_hip_device* dev, const MatmulCall& call);
 
+// matmul_skinny.hip: at most 16 columns and 1024 rows of C, both operands as
+// stored, K a multiple of 4 and at most 16384: one wave per row of C, one launch.
+bool skinnyMatmulApplies(const MatmulCall& call);
+int launchSkinnyMatmul(polar_hip_device* dev, const MatmulCall& call);
+
 } // namespace polar_hip_detail

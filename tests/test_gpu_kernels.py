@@ -304,11 +304,48 @@ def test_matmul_split_contraction_is_added_by_the_last_group_repeatably(dev):
         t.free()
 
 
+SKINNY_SHAPES = [(256, 10, 784), (1, 1, 64), (1, 1, 16384), (7, 3, 100), (300, 16, 68), (512, 1, 16384),
+                 (1000, 5, 260), (64, 8, 1024), (2, 13, 1260), (1024, 1, 64), (1024, 10, 784), (16, 16, 1024),
+                 # not this kernel's (K no multiple of 4, K too short, too many rows or columns, too much of B):
+                 # passed on
+                 (256, 10, 786), (256, 10, 60), (1025, 10, 784), (256, 17, 784), (1024, 16, 784), (513, 9, 4096)]
+
+
+@pytest.mark.parametrize("mnk", SKINNY_SHAPES)
+def test_matmul_with_a_skinny_result(dev, mnk):
+    """At most 16 columns and 1024 rows of C, operands as stored: one wave per row of C
+    in one launch (the logistic-regression forward product).  Integer data is exact
+    under any order of the additions; bases off 16 bytes go to the tiled kernel."""
+    m, n, k = mnk
+    rng = np.random.default_rng(4100 + m + n + k)
+    a = rng.integers(-8, 9, (m, k)).astype(np.float32)
+    b = rng.integers(-8, 9, (k, n)).astype(np.float32)
+    ref = o.fmatmul(False, False, a, b)
+    for mis_a, mis_b, mis_c in ((0, 0, 0), (0, 0, 5), (1, 0, 0), (0, 3, 2)):
+        _say("skinny matmul", mnk, "misalign", (mis_a, mis_b, mis_c), "plan", dev.fmatmul_plan(m, n, k))
+        da, db, dc = dev.array(a, mis_a), dev.array(b, mis_b), dev.empty(m * n + 32, mis_c)
+        dev.ffill(-7.0, dc)
+        dev.fmatmul(False, False, da, db, dc, m, n, k)
+        got = dc.download()
+        assert np.array_equal(got[:m * n].reshape(m, n), ref)
+        assert np.all(got[m * n:] == -7.0)
+        for t in (da, db, dc):
+            t.free()
+    # real-valued data against the oracle's sequential sum
+    a, b = parity.normal(rng, (m, k)), parity.normal(rng, (k, n))
+    da, db, dc = dev.array(a), dev.array(b), dev.empty(m * n)
+    dev.fmatmul(False, False, da, db, dc, m, n, k)
+    assert parity.frobenius_rel_error(dc.download((m, n)), o.fmatmul(False, False, a, b)) <= parity.MATMUL_FRO_REL
+    for t in (da, db, dc):
+        t.free()
+
+
 def test_matmul_plan_is_reported_and_forced_plans_are_checked(dev):
     config, splits, tile = dev.fmatmul_plan(4096, 4096, 4096)
     assert (config, splits, tile) == (0, 1, (256, 256, 32))
-    config, splits, tile = dev.fmatmul_plan(256, 10, 784)
+    config, splits, tile = dev.fmatmul_plan(300, 257, 3000)
     assert 0 <= config < 10 and splits > 1 and tile[2] == 32
+    assert dev.fmatmul_plan(256, 10, 784)[0] == -1            # one wave per row of a skinny result
     assert dev.fmatmul_plan(65536, 33, 127)[0] == -1          # the short-contraction kernels
     x, y, z = dev.empty(64 * 64), dev.empty(64 * 64), dev.empty(64 * 64)
     for bad in ((10, 1), (-1, 1), (2, 0), (2, 257)):
